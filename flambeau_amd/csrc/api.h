@@ -313,6 +313,39 @@ int fl_rotate_scale(const float* proj, int ld, int col_a, int col_b, const float
                     float scale_a, float scale_b, float* out_a, float* out_b, int n, int H, int D,
                     hipStream_t stream);
 
+// ---- layer norm, learned positions, forget gates per key dim, attention whose heads' scores are mixed ----
+// out = (v - mean) / sqrt(var + eps) * w + b of v = x (+ delta); resid_out, rows as for fl_rmsnorm; b may be null
+int fl_layernorm(const float* x, const float* delta, float* resid_out, const int* rows, const float* w,
+                 const float* b, void* out, int out_dtype, int n, int H, float eps, hipStream_t stream);
+// resid += layernorm(delta); cast (or null) receives the new resid in cast_dtype
+int fl_layernorm_add(const float* delta, const float* w, const float* b, float* resid, void* cast, int cast_dtype,
+                     int n, int H, float eps, hipStream_t stream);
+// out[t] = table[tokens[t]] + pos_table[positions[t]] (both tables in dtype, the sum float)
+int fl_embed_positions(const void* table, const void* pos_table, int dtype, const int* tokens, const int* positions,
+                       float* out, int n, int H, int V, int P, hipStream_t stream);
+int fl_cast_rows(const float* x, void* out, int out_dtype, long total, hipStream_t stream);
+int fl_scale_inplace(float* x, long total, float s, hipStream_t stream);
+// out[r][i] = act(x[r][i] + bias[i]); kinds as fl_activation (3: the square of relu)
+int fl_bias_activation(const float* x, const float* bias, void* out, int out_dtype, int n, int width, int kind,
+                       hipStream_t stream);
+// fl_linear_scan with a forget gate f per token, head and key dim: S <- diag(f) S + (1 - f) v^T, o = S^T q
+int fl_linear_scan_channel(const float* q, int ldq, const float* f, int ldf, const float* v, int ldv, float* state,
+                           long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                           float* out, int n_seqs, int H, int D, int Dv, hipStream_t stream);
+// q_out = silu(proj[col_q ..]), f_out = lower + (1 - lower) * sigmoid(proj[col_f ..] + bias), HD values per row
+int fl_forget_gates(const float* proj, int ld, int col_q, int col_f, const float* bias, const float* lower,
+                    float* q_out, float* f_out, int n, int HD, hipStream_t stream);
+// Softmax attention over the paged cache with a distance bias slope_g * (i - j) taken off every head's score,
+// the heads' scores mixed by talk [nh][nh], and a sink per head in the denominator (each may be null).
+// part_keys > 0: a token's keys are dealt out to n_parts blocks of part_keys keys and joined afterwards
+// (part_acc [n][n_parts][nh][hd], part_ml [n][n_parts][nh][2], float).
+int fl_attn_mixed_max_heads(int hd);
+int fl_attn_mixed(const void* q, void* out, const void* cache_base, int dtype, const int* positions,
+                  const int* tok_seq, const int* block_table, int max_blocks, int n, int nh, int nkv, int hd,
+                  int page_size, int n_pages, float scale, int window, const float* slopes, const float* talk,
+                  const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
+                  hipStream_t stream);
+
 // ---- step programs (program.hip): launches recorded once, replayed with one call ----
 typedef union FlArg { void* p; long l; int i; float f; } FlArg;
 void* fl_program_new(void);

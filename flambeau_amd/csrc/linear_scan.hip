@@ -35,7 +35,9 @@
 // The step's tokens come through LDS a run of RUN tokens at a time, rows 16 * RPT wide and zero behind D;
 // the next run's values are asked for (into registers) before the walk over this run begins and put into
 // LDS after it, so that the trip to memory hides behind the walk.
-template <int RPT, bool DELTA>
+// MODE 0: a decay per head or per token and head, u = v; 1: the delta rule; 2: a decay per token, head AND key dim
+// (`k` holds the forget gates f; the key is 1 - f: what is forgotten makes room for what is written)
+template <int RPT, int MODE>
 __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ head_decay, const float* __restrict__ tok_decay, const float* __restrict__ beta, int ldg,
@@ -72,7 +74,7 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
             const bool in = tt < cnt && d < D;
             const size_t row = (size_t)(start + t0 + (in ? tt : 0));
             pq[i] = in ? q[row * ldq + qk_head * D + d] : 0.f;
-            pk[i] = in ? k[row * ldk + qk_head * D + d] : 0.f;
+            pk[i] = in ? k[row * ldk + qk_head * D + d] : (MODE == 2 ? 1.f : 0.f);
         }
 #pragma unroll
         for (int i = 0; i < PRE_V; ++i) {
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
         if (threadIdx.x < cnt) {
             const size_t row = (size_t)(start + t0 + threadIdx.x);
             pf0 = tok_decay ? tok_decay[row * ldg + head] : fixed;
-            pf1 = DELTA ? beta[row * ldg + head] : 1.f;
+            pf1 = MODE == 1 ? beta[row * ldg + head] : 1.f;
         }
     };
     if (len > 0) fetch(0);
@@ -110,9 +112,14 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
             for (int u = 0; u < RPT; ++u) {
                 kr[u] = ks[tt * DP + g * RPT + u];
                 qr[u] = qs[tt * DP + g * RPT + u];
-                S[u] *= decay;
+                if (MODE == 2) {
+                    S[u] *= kr[u];
+                    kr[u] = 1.0f - kr[u];
+                } else {
+                    S[u] *= decay;
+                }
             }
-            if (DELTA) {
+            if (MODE == 1) {
                 float seen0 = 0.f, seen1 = 0.f;                   // two chains of half the length
 #pragma unroll
                 for (int u = 0; u < RPT; u += 2) {
@@ -144,28 +151,30 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
 
 extern "C" int fl_linear_scan_max_dim(void) { return LS_GROUP * LS_MAX_ROWS; }
 
-extern "C" int fl_linear_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+static int linear_scan_launch(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                               const float* head_decay, const float* tok_decay, const float* beta, int ldg, float* state,
                               long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
-                              float* out, int n_seqs, int H, int G, int D, int Dv, hipStream_t stream) {
+                              float* out, int n_seqs, int H, int G, int D, int Dv, bool channel_decay, hipStream_t stream) {
     FL_CHECK(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0, "linear_scan: bad sizes");
     FL_CHECK(D <= LS_GROUP * LS_MAX_ROWS, "linear_scan: %d key dims per head, at most %d", D, LS_GROUP * LS_MAX_ROWS);
     FL_CHECK(ldq >= G * D && ldk >= G * D && ldv >= H * Dv, "linear_scan: rows narrower than their heads");
-    FL_CHECK(!head_decay != !tok_decay, "linear_scan: one decay per head or one per token and head, not both or none");
+    FL_CHECK(channel_decay ? (!head_decay && !tok_decay && !beta && H == G)
+                           : (!head_decay != !tok_decay), "linear_scan: one decay per head, or one per token and head, or one per token, head and key dim");
     FL_CHECK((!tok_decay && !beta) || ldg >= H, "linear_scan: gate rows %d wide for %d heads", ldg, H);
     FL_CHECK(slot_stride >= (long)H * D * Dv, "linear_scan: a slot of %ld floats does not hold %d heads", slot_stride, H);
     if (n_seqs == 0) return 0;
     FL_CHECK(n_seqs <= 65535 && H <= 65535, "linear_scan: %d requests of %d heads are more than one grid takes", n_seqs, H);
     dim3 grid(ceil_div(Dv, LS_COLS), H, n_seqs);
     const int rpt = ceil_div(D, LS_GROUP);
-#define FL_LS2(R, DELTA)                                                                                              \
-    linear_scan_kernel<R, DELTA><<<grid, LS_GROUP * LS_COLS, 0, stream>>>(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, \
+#define FL_LS2(R, MODE)                                                                                               \
+    linear_scan_kernel<R, MODE><<<grid, LS_GROUP * LS_COLS, 0, stream>>>(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, \
                                                                           ldg, state, (size_t)slot_stride, seq_q_start,        \
                                                                           seq_q_len, seq_slots, out, H, G, D, Dv)
 #define FL_LS(R)             \
     do {                     \
-        if (beta) FL_LS2(R, true); \
-        else FL_LS2(R, false);     \
+        if (channel_decay) FL_LS2(R, 2); \
+        else if (beta) FL_LS2(R, 1);     \
+        else FL_LS2(R, 0);               \
     } while (0)
     if (rpt <= 1) FL_LS(1);
     else if (rpt <= 2) FL_LS(2);
@@ -178,7 +187,49 @@ extern "C" int fl_linear_scan(const float* q, int ldq, const float* k, int ldk, 
     FL_LAUNCH_CHECK();
     return 0;
 }
+
+extern "C" int fl_linear_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                              const float* head_decay, const float* tok_decay, const float* beta, int ldg, float* state,
+                              long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                              float* out, int n_seqs, int H, int G, int D, int Dv, hipStream_t stream) {
+    return linear_scan_launch(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, ldg, state, slot_stride, seq_q_start,
+                              seq_q_len, seq_slots, out, n_seqs, H, G, D, Dv, false, stream);
+}
 FL_RECORDABLE(fl_linear_scan)
+
+// The same walk with a forget gate per token, head and key dim: S <- diag(f) S + (1 - f) v^T, o = S^T q.
+extern "C" int fl_linear_scan_channel(const float* q, int ldq, const float* f, int ldf, const float* v, int ldv, float* state,
+                                      long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
+                                      float* out, int n_seqs, int H, int D, int Dv, hipStream_t stream) {
+    return linear_scan_launch(q, ldq, f, ldf, v, ldv, nullptr, nullptr, nullptr, 0, state, slot_stride, seq_q_start,
+                              seq_q_len, seq_slots, out, n_seqs, H, H, D, Dv, true, stream);
+}
+FL_RECORDABLE(fl_linear_scan_channel)
+
+// What stands between the joined projection of a mixer with forget gates per key dim and its walk:
+// q = silu(q), f = lower + (1 - lower) * sigmoid(f + bias), both float, value by value.
+__global__ __launch_bounds__(256) void forget_gates_kernel(const float* __restrict__ proj, int ld, int col_q, int col_f,
+                                                           const float* __restrict__ bias, const float* __restrict__ lower,
+                                                           float* __restrict__ q_out, float* __restrict__ f_out, int HD) {
+    const float* row = proj + (size_t)blockIdx.x * ld;
+    for (int i = threadIdx.x; i < HD; i += 256) {
+        const float zq = row[col_q + i];
+        q_out[(size_t)blockIdx.x * HD + i] = zq / (1.0f + expf(-zq));
+        const float low = lower ? lower[i] : 0.f;
+        const float zf = row[col_f + i] + (bias ? bias[i] : 0.f);
+        f_out[(size_t)blockIdx.x * HD + i] = low + (1.0f - low) / (1.0f + expf(-zf));
+    }
+}
+
+extern "C" int fl_forget_gates(const float* proj, int ld, int col_q, int col_f, const float* bias, const float* lower,
+                               float* q_out, float* f_out, int n, int HD, hipStream_t stream) {
+    FL_CHECK(n >= 0 && HD > 0 && ld >= col_q + HD && ld >= col_f + HD && col_q >= 0 && col_f >= 0, "forget_gates: columns beyond rows %d wide", ld);
+    if (n == 0) return 0;
+    forget_gates_kernel<<<n, 256, 0, stream>>>(proj, ld, col_q, col_f, bias, lower, q_out, f_out, HD);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_forget_gates)
 
 // ------------------------------------------------------------------ short convolution, unit vectors, gates
 struct ConvPrepare {

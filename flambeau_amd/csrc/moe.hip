@@ -18,7 +18,8 @@
 #define MOE_MAX_TOP 16
 
 // logits: float rows ld wide, the experts' at col0 .. col0 + E - 1.  kind 0: weight = sigmoid(logit);
-// kind 1: weight = softmax over all experts.  renorm: the chosen weights are divided by their sum.
+// kind 1: weight = softmax over all experts; kind 2: softmax over the chosen logits only.  renorm: the chosen
+// weights are divided by their sum (kind 2 always).
 // place [n * top]: where pair (t, k) lies in the sorted order; src_row / src_scale [n * top]: token and weight
 // of every sorted place; tiles [max_tiles][4] = (expert, first place, places, 0), expert -1: unused.
 __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__ logits, int ld, int col0, int n, int E,
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
             zsum = wave_sum(zsum);
         }
         int chosen[MOE_MAX_TOP];
-        float w[MOE_MAX_TOP], wsum = 0.f;
+        float w[MOE_MAX_TOP], wsum = 0.f, zfirst = 0.f;
         for (int k = 0; k < top; ++k) {
             float bz = -INFINITY;
             int best = 0x7fffffff;
@@ -70,13 +71,14 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
             for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
                 if (u < nu && lane + 64 * u == best) zv[u] = -INFINITY;      // taken
             chosen[k] = best;
-            w[k] = kind == 1 ? expf(bz - zmax) / zsum : 1.0f / (1.0f + expf(-bz));
+            if (k == 0) zfirst = bz;                              // the largest logit
+            w[k] = kind == 2 ? expf(bz - zfirst) : kind == 1 ? expf(bz - zmax) / zsum : 1.0f / (1.0f + expf(-bz));
             wsum += w[k];
         }
         if (lane == 0) {
             for (int k = 0; k < top; ++k) {
                 place[(size_t)t * top + k] = chosen[k];
-                pair_w[(size_t)t * top + k] = renorm ? w[k] / wsum : w[k];
+                pair_w[(size_t)t * top + k] = (renorm || kind == 2) ? w[k] / wsum : w[k];
             }
         }
     }
@@ -134,7 +136,7 @@ extern "C" int fl_moe_route(const float* logits, int ld, int col0, int n, int E,
         const long pairs = (long)n * top;          // an expert's last tile may be short: pairs / 64 full tiles and one per expert at most
         FL_CHECK((long)max_tiles >= pairs / MOE_TILE + (pairs < E ? pairs : E), "moe_route: %d tiles cannot hold %ld rows of %d experts", max_tiles, pairs, E);
     }
-    FL_CHECK(kind == 0 || kind == 1, "moe_route: unknown scoring %d", kind);
+    FL_CHECK(kind >= 0 && kind <= 2, "moe_route: unknown scoring %d", kind);
     if (n == 0) return 0;
     const int pick_blocks = n < 4 * 1024 ? (n + 3) / 4 : 1024;
     moe_pick_kernel<<<pick_blocks, 256, 0, stream>>>(logits, ld, col0, n, E, top, kind, renorm, place, pair_w);
@@ -277,19 +279,21 @@ FL_RECORDABLE(fl_moe_combine)
 // kind 0: gelu with the error function, 0.5 z (1 + erf(z / sqrt 2)); 1: its tanh form,
 // 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))); 2: silu, z / (1 + exp(-z)).
 template <typename TOut>
-__global__ __launch_bounds__(256) void activation_kernel(const float* __restrict__ x, TOut* __restrict__ out, long total, int kind) {
+__global__ __launch_bounds__(256) void activation_kernel(const float* __restrict__ x, TOut* __restrict__ out, long total, int kind,
+                                                         const float* __restrict__ bias = nullptr, int width = 1) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
-    const float z = x[i];
+    const float z = bias ? x[i] + bias[i % width] : x[i];
     float y;
     if (kind == 0) y = 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
     else if (kind == 1) y = 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+    else if (kind == 3) y = z > 0.f ? z * z : 0.f;
     else y = z / (1.0f + expf(-z));
     out[i] = from_f32<TOut>(y);
 }
 
 extern "C" int fl_activation(const float* x, void* out, int out_dtype, long total, int kind, hipStream_t stream) {
-    FL_CHECK(total >= 0 && kind >= 0 && kind <= 2, "activation: bad size or kind %d", kind);
+    FL_CHECK(total >= 0 && kind >= 0 && kind <= 3, "activation: bad size or kind %d", kind);
     if (total == 0) return 0;
     const unsigned blocks = (unsigned)((total + 255) / 256);
     if (out_dtype == FL_F32) activation_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, total, kind);
@@ -299,6 +303,21 @@ extern "C" int fl_activation(const float* x, void* out, int out_dtype, long tota
     return 0;
 }
 FL_RECORDABLE(fl_activation)
+
+// out[r][i] = act(x[r][i] + bias[i]): the activation of a feed-forward whose first product has a bias
+extern "C" int fl_bias_activation(const float* x, const float* bias, void* out, int out_dtype, int n, int width, int kind,
+                                  hipStream_t stream) {
+    FL_CHECK(n >= 0 && width > 0 && kind >= 0 && kind <= 3 && bias, "bias_activation: bad size, kind %d or no bias", kind);
+    const long total = (long)n * width;
+    if (total == 0) return 0;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (out_dtype == FL_F32) activation_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, total, kind, bias, width);
+    else if (out_dtype == FL_BF16) activation_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, (bf16_t*)out, total, kind, bias, width);
+    else FL_CHECK(false, "bias_activation: unknown dtype %d", out_dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_bias_activation)
 
 // ------------------------------------------------------------------ re-entry of the residual stream
 // out[r] = [a[r] ; b[r]] in the storage type (two float rows of W values side by side).

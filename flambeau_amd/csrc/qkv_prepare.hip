@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void qkv_row_scales_kernel(QkvPrepare a, int n
     const float* row = a.proj + (size_t)blockIdx.x * a.ld;
     float sq = 0.f, sk = 0.f;
     for (int i = threadIdx.x; i < a.nh * a.D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
-    for (int i = threadIdx.x; i < nkv * a.D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
+    if (a.col_k >= 0) for (int i = threadIdx.x; i < nkv * a.D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
     sq = block_sum<4>(sq, lds);
     sk = block_sum<4>(sk, lds + 4);
     if (threadIdx.x == 0) {
@@ -49,6 +49,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     const int token = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nh = a.nh, nkv = cache.n_kv_heads, D = a.D, Dv = a.Dv, hdp = a.hdp;
     const float* row = a.proj + (size_t)token * a.ld;
+    const bool has_kv = a.col_k >= 0;                 // (a mixer that reads another layer's keys and values projects queries alone)
     float inv_q = 1.f, inv_k = 1.f;
     if (a.qnorm_w && a.row_scales) {
         inv_q = a.row_scales[2 * token];
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
         // (a step of few tokens: every block sums for itself, in the same order as the kernel above, and a launch is saved)
         float sq = 0.f, sk = 0.f;
         for (int i = threadIdx.x; i < nh * D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
-        for (int i = threadIdx.x; i < nkv * D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
+        if (has_kv) for (int i = threadIdx.x; i < nkv * D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
         inv_q = 1.0f / sqrtf(block_sum<4>(sq, lds) / (float)(nh * D) + a.eps);
         inv_k = 1.0f / sqrtf(block_sum<4>(sk, lds + 4) / (float)(nkv * D) + a.eps);
     }
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     // q and k heads: a wave per head, a lane per head dim (and the dims 64, 128, ... further); the heads of a token
     // are spread over blocks of four waves (every block forms the projection's sums of squares for itself)
     const int head = blockIdx.y * 4 + wave;
-    if (head < nh + nkv) {
+    if (head < nh + (has_kv ? nkv : 0)) {
         const bool is_q = head < nh;
         const int h = is_q ? head : head - nh;
         const float* src = row + (is_q ? a.col_q : a.col_k) + h * D;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     }
     // v heads: the blocks share their values out
     const float lam = a.vmix_mode == 2 ? a.lambda[0] : 0.f;
-    for (int e = blockIdx.y * 256 + threadIdx.x; e < nkv * hdp; e += 256 * gridDim.y) {
+    for (int e = blockIdx.y * 256 + threadIdx.x; has_kv && e < nkv * hdp; e += 256 * gridDim.y) {
         const int h = e / hdp, d = e - h * hdp;
         float v = 0.f;
         if (d < Dv) {
@@ -141,8 +142,9 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
     FL_CHECK(hdp >= D && hdp >= Dv && hdp <= 256, "qkv_prepare: heads of %d and %d values stored %d wide (at most 256)", D, Dv, hdp);
     FL_CHECK(rot >= 0 && rot <= D && rot % 2 == 0, "qkv_prepare: rotated dims %d of head %d", rot, D);
     FL_CHECK(rot == 0 || cs, "qkv_prepare: a rotation needs the step's table of cosines and sines");
-    FL_CHECK(ld >= col_q + nh * D && ld >= col_k + nkv * D && ld >= col_v + nkv * Dv, "qkv_prepare: columns beyond rows %d wide", ld);
-    FL_CHECK(!qnorm_w == !knorm_w, "qkv_prepare: the norm over the projection needs both gains");
+    FL_CHECK(ld >= col_q + nh * D && (col_k < 0 || (ld >= col_k + nkv * D && ld >= col_v + nkv * Dv)), "qkv_prepare: columns beyond rows %d wide", ld);
+    FL_CHECK(col_k >= 0 || !write_cache, "qkv_prepare: a projection of queries alone writes no cache");
+    FL_CHECK(col_k < 0 ? !knorm_w : !qnorm_w == !knorm_w, "qkv_prepare: the norm over the projection needs both gains");
     FL_CHECK(vmix_mode >= 0 && vmix_mode <= 2 && (vmix_mode == 0 || v_first) && (vmix_mode != 2 || lambda),
              "qkv_prepare: value blending %d without its buffers", vmix_mode);
     if (n == 0) return 0;
@@ -150,7 +152,7 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
                  rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, v_first, vmix_mode, lambda, write_cache,
                  (qnorm_w && n > QKV_FEW_TOKENS) ? row_scales : nullptr};
     PagedCache c{cache_base, nkv, page_size, hdp, n_pages};
-    dim3 grid(n, ceil_div(nh + nkv, 4));
+    dim3 grid(n, ceil_div(nh + (col_k >= 0 ? nkv : 0), 4));
     FL_CHECK(grid.y <= 65535, "qkv_prepare: %d heads are more than one grid takes", nh + nkv);
     if (a.row_scales) {
         // many tokens: the sums of squares once per token, not once per block of four heads

@@ -60,6 +60,15 @@ _SIGNATURES = {
     "fl_linear_scan": [P, I, P, I, P, I, P, P, P, I, P, L, P, P, P, P, I, I, I, I, I, P],
     "fl_conv_prepare": [P, I, I, I, I, P, P, P, P, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P],
     "fl_rotate_scale": [P, I, I, I, P, I, I, F, F, P, P, I, I, I, P],
+    "fl_layernorm": [P, P, P, P, P, P, P, I, I, I, F, P],
+    "fl_layernorm_add": [P, P, P, P, P, I, I, I, F, P],
+    "fl_embed_positions": [P, P, I, P, P, P, I, I, I, I, P],
+    "fl_cast_rows": [P, P, I, L, P],
+    "fl_scale_inplace": [P, L, F, P],
+    "fl_bias_activation": [P, P, P, I, I, I, I, P],
+    "fl_linear_scan_channel": [P, I, P, I, P, I, P, L, P, P, P, P, I, I, I, I, P],
+    "fl_forget_gates": [P, I, I, I, P, P, P, P, I, I, P],
+    "fl_attn_mixed": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, P, I, I, P, P, P],
 }
 
 

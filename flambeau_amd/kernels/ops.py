@@ -409,13 +409,19 @@ def headnorm_gate(x, weight, gate, gate_col0, out, n_heads, eps, gate_kind: str 
     return out
 
 
-ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu2": 3}
 
 
-def activation(x, out, kind: str):
-    """``out = act(x)`` for float32 ``x``: ``gelu`` (with the error function), ``gelu_tanh``, ``silu``."""
+def activation(x, out, kind: str, bias=None):
+    """``out = act(x (+ bias))`` for float32 ``x``: ``gelu`` (with the error function), ``gelu_tanh``, ``silu``,
+    ``relu2`` (the square of relu); ``bias``: float32, one value per column."""
     if x.shape != out.shape:
         raise KernelError(f"activation: shapes {tuple(x.shape)} and {tuple(out.shape)} differ")
+    if bias is not None:
+        n, F = x.shape
+        call("fl_bias_activation", _check(x, "activation.x", torch.float32), _check(bias, "activation.bias", torch.float32, (F,)),
+             _check(out, "activation.out"), dtype_code(out.dtype), n, F, ACTIVATIONS[kind], stream_handle())
+        return out
     call("fl_activation", _check(x, "activation.x", torch.float32), _check(out, "activation.out"), dtype_code(out.dtype),
          x.numel(), ACTIVATIONS[kind], stream_handle())
     return out
@@ -431,11 +437,14 @@ def moe_max_tiles(n_pairs: int, n_experts: int) -> int:
     return n_pairs // moe_tile_rows() + min(n_pairs, n_experts)
 
 
+ROUTER_SCORINGS = {"sigmoid": 0, "softmax": 1, "softmax_chosen": 2}
+
+
 def moe_route(logits, col0, n_experts, top, place, src_row, src_scale, pair_w, tiles, scoring="sigmoid", renormalise=False):
     n, ld = logits.shape
     P_ = n * top
     call("fl_moe_route", _check(logits, "moe_route.logits", torch.float32), ld, int(col0), n, int(n_experts), int(top),
-         {"sigmoid": 0, "softmax": 1}[scoring], int(bool(renormalise)),
+         ROUTER_SCORINGS[scoring], int(bool(renormalise)),
          _check(place, "moe_route.place", torch.int32, (P_,)), _check(src_row, "moe_route.src_row", torch.int32, (P_,)),
          _check(src_scale, "moe_route.src_scale", torch.float32, (P_,)), _check(pair_w, "moe_route.pair_w", torch.float32, (P_,)),
          _check(tiles, "moe_route.tiles", torch.int32, (None, 4)), tiles.shape[0], stream_handle())
@@ -571,6 +580,8 @@ def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: Paged
     nkv, hdp = cache.n_kv_heads, cache.head_dim
     dt = cache.pool.dtype
     half = rotated_dims // 2
+    if cols[1] < 0 and write_cache:
+        raise KernelError("qkv_prepare: a projection of queries alone (no key columns) writes no cache")
     call("fl_qkv_prepare", _check(proj, "qkv_prepare.proj", torch.float32), ld, *(int(c) for c in cols),
          _check(positions, "qkv_prepare.positions", torch.int32, (n,)), _check(tok_seq, "qkv_prepare.tok_seq", torch.int32, (n,)),
          _check(block_table, "qkv_prepare.block_table", torch.int32, (None, None)), block_table.shape[1],
@@ -597,12 +608,13 @@ def conv_max_taps() -> int:
 
 
 def linear_scan(q, k, v, state, seq_q_start, seq_q_len, seq_slots, out, n_heads, n_qk_heads, dim, vdim,
-                head_decay=None, token_gates=None):
+                head_decay=None, token_gates=None, channel_decay: bool = False):
     """The recurrence S <- g S + k u^T, o = S^T q over the step's tokens, request by request, from and into
     the first ``heads * dim * vdim`` floats of every slot's record in ``state`` ``[slots, floats]``.
     ``q``, ``k`` float32 ``[n, n_qk_heads * dim]`` (views of wider rows are taken with their row stride),
     ``v`` ``[n, n_heads * vdim]``.  ``head_decay`` float32 ``[heads]``: a fixed g per head and u = v;
-    ``token_gates`` float32 ``[n, 2 * heads]`` (g, then beta): the delta rule, u = beta (v - S^T k)."""
+    ``token_gates`` float32 ``[n, 2 * heads]`` (g, then beta): the delta rule, u = beta (v - S^T k).
+    ``channel_decay``: ``k`` holds a forget gate f per token, head and key dim, S <- diag(f) S + (1 - f) v^T."""
     n = out.shape[0]
     S = seq_q_start.shape[0]
     if state.dim() != 2 or not state.is_contiguous():
@@ -613,6 +625,14 @@ def linear_scan(q, k, v, state, seq_q_start, seq_q_len, seq_slots, out, n_heads,
             raise KernelError(f"linear_scan.{name}: {t.dtype} {tuple(t.shape)}, want float32 [{n}, {width}] with unit stride")
         return t.data_ptr(), t.stride(0)
     (pq, ldq), (pk, ldk), (pv, ldv) = rows(q, "q", n_qk_heads * dim), rows(k, "k", n_qk_heads * dim), rows(v, "v", n_heads * vdim)
+    if channel_decay:
+        if head_decay is not None or token_gates is not None or n_heads != n_qk_heads:
+            raise KernelError("linear_scan: forget gates per key dim come alone, one set per head")
+        call("fl_linear_scan_channel", pq, ldq, pk, ldk, pv, ldv, _check(state, "linear_scan.state", torch.float32), state.shape[1],
+             _check(seq_q_start, "linear_scan.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "linear_scan.seq_q_len", torch.int32, (S,)),
+             _check(seq_slots, "linear_scan.seq_slots", torch.int32, (S,)), _check(out, "linear_scan.out", torch.float32, (n, n_heads * vdim)),
+             S, int(n_heads), int(dim), int(vdim), stream_handle())
+        return out
     if (head_decay is None) == (token_gates is None):
         raise KernelError("linear_scan: a decay per head or gates per token, one of the two")
     pg = _check(token_gates, "linear_scan.gates", torch.float32, (n, 2 * n_heads)) if token_gates is not None else None
@@ -657,3 +677,97 @@ def rotate_scale(proj, col_a, col_b, table, rotated_dims, interleaved, scale_a, 
          int(rotated_dims), int(bool(interleaved)), float(scale_a), float(scale_b),
          _check(out_a, "rotate_scale.out_a", torch.float32, (n, n_heads * dim)),
          _check(out_b, "rotate_scale.out_b", torch.float32, (n, n_heads * dim)), n, int(n_heads), int(dim), stream_handle())
+
+
+# ---------------------------------------------------------------- layer norm, learned positions, forget gates, mixed heads
+def layernorm(x, weight, bias, out, eps, delta=None, store_sum=False, rows=None):
+    """``out = layernorm(x (+ delta)) * weight + bias`` (mean and variance over a row); ``store_sum`` and ``rows``
+    as for ``rmsnorm``; ``out`` may be ``x`` itself."""
+    n, H = x.shape
+    px = _check(x, "layernorm.x", torch.float32, (n, H))
+    pd = _check(delta, "layernorm.delta", torch.float32, (n, H)) if delta is not None else None
+    pr = _check(rows, "layernorm.rows", torch.int32) if rows is not None else None
+    n_out = rows.shape[0] if rows is not None else n
+    call("fl_layernorm", px, pd, px if store_sum and delta is not None else None, pr,
+         _check(weight, "layernorm.weight", torch.float32, (H,)),
+         _check(bias, "layernorm.bias", torch.float32, (H,)) if bias is not None else None,
+         _check(out, "layernorm.out", None, (n_out, H)), dtype_code(out.dtype), n_out, H, float(eps), stream_handle())
+    return out
+
+
+def layernorm_add(delta, weight, bias, resid, eps, cast=None):
+    """``resid += layernorm(delta) * weight + bias``; ``cast`` (optional) receives the new ``resid`` in its dtype."""
+    n, H = resid.shape
+    call("fl_layernorm_add", _check(delta, "layernorm_add.delta", torch.float32, (n, H)),
+         _check(weight, "layernorm_add.weight", torch.float32, (H,)),
+         _check(bias, "layernorm_add.bias", torch.float32, (H,)) if bias is not None else None,
+         _check(resid, "layernorm_add.resid", torch.float32),
+         _check(cast, "layernorm_add.cast", None, (n, H)) if cast is not None else None,
+         dtype_code(cast.dtype) if cast is not None else 0, n, H, float(eps), stream_handle())
+    return resid
+
+
+def embed_positions(table, pos_table, tokens, positions, out):
+    """``out[t] = table[tokens[t]] + pos_table[positions[t]]`` in float32."""
+    V, H = table.shape
+    P_ = pos_table.shape[0]
+    n = tokens.shape[0]
+    call("fl_embed_positions", _check(table, "embed.table"), _check(pos_table, "embed.pos_table", table.dtype, (P_, H)),
+         dtype_code(table.dtype), _check(tokens, "embed.tokens", torch.int32, (n,)),
+         _check(positions, "embed.positions", torch.int32, (n,)), _check(out, "embed.out", torch.float32, (n, H)),
+         n, H, V, P_, stream_handle())
+    return out
+
+
+def cast_rows(x, out):
+    """The float32 ``x`` in ``out``'s dtype."""
+    if x.shape != out.shape:
+        raise KernelError(f"cast_rows: shapes {tuple(x.shape)} and {tuple(out.shape)} differ")
+    call("fl_cast_rows", _check(x, "cast_rows.x", torch.float32), _check(out, "cast_rows.out"), dtype_code(out.dtype),
+         x.numel(), stream_handle())
+    return out
+
+
+def scale_inplace(x, factor: float):
+    call("fl_scale_inplace", _check(x, "scale.x", torch.float32), x.numel(), float(factor), stream_handle())
+    return x
+
+
+def forget_gates(proj, col_q, col_f, bias, lower, q_out, f_out):
+    """``q_out = silu(proj[:, col_q:])``, ``f_out = lower + (1 - lower) * sigmoid(proj[:, col_f:] + bias)``, float32
+    ``[n, HD]`` each: the read-out vector and the forget gates of a recurrence whose gate is also its key."""
+    n, ld = proj.shape
+    HD = q_out.shape[1]
+    call("fl_forget_gates", _check(proj, "forget_gates.proj", torch.float32), ld, int(col_q), int(col_f),
+         _check(bias, "forget_gates.bias", torch.float32, (HD,)) if bias is not None else None,
+         _check(lower, "forget_gates.lower", torch.float32, (HD,)) if lower is not None else None,
+         _check(q_out, "forget_gates.q", torch.float32, (n, HD)), _check(f_out, "forget_gates.f", torch.float32, (n, HD)),
+         n, HD, stream_handle())
+
+
+def attn_mixed_max_heads(head_dim: int) -> int:
+    """How many heads of ``head_dim`` stored values a block of the mixed-heads attention kernel holds."""
+    from .library import load
+    return load().fl_attn_mixed_max_heads(int(head_dim))
+
+
+def attn_mixed(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, n_heads, scale, window,
+               slopes=None, talk=None, sink=None, part_keys: int = 0, n_parts: int = 1, part_acc=None, part_ml=None):
+    """Attention over the paged cache with ``slopes[g] * (i - j)`` taken off the scores, the heads' scores mixed by
+    ``talk`` ``[H, H]`` and ``exp(sink[h])`` in the denominator (each optional).  ``part_keys`` > 0: every
+    token's keys are dealt out to ``n_parts`` blocks; ``part_acc`` / ``part_ml`` float32 scratch for them."""
+    n = q.shape[0]
+    hd = cache.head_dim
+    dt = cache.pool.dtype
+    f = lambda t, name, shape: _check(t, "attn_mixed." + name, torch.float32, shape) if t is not None else None
+    if part_keys:
+        if part_acc is None or part_ml is None or part_acc.numel() < n * n_parts * n_heads * hd or part_ml.numel() < n * n_parts * n_heads * 2:
+            raise KernelError("attn_mixed: the parts' scratch is missing or too small")
+    call("fl_attn_mixed", _check(q, "attn_mixed.q", dt, (n, n_heads * hd)), _check(out, "attn_mixed.out", dt, (n, n_heads * hd)),
+         _check(cache.pool, "attn_mixed.cache"), dtype_code(dt), _check(positions, "attn_mixed.positions", torch.int32, (n,)),
+         _check(tok_seq, "attn_mixed.tok_seq", torch.int32, (n,)),
+         _check(block_table, "attn_mixed.block_table", torch.int32, (None, None)), block_table.shape[1],
+         n, int(n_heads), cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window),
+         f(slopes, "slopes", (n_heads,)), f(talk, "talk", (n_heads, n_heads)), f(sink, "sink", (n_heads,)),
+         int(part_keys), int(n_parts), f(part_acc, "part_acc", None), f(part_ml, "part_ml", None), stream_handle())
+    return out

@@ -196,10 +196,11 @@ class DecoderModel:
         rt = self.rt
         step.scratch.clear()
         resid = rt.buffer("residual", step.n_tokens, self.spec.hidden_size, torch.float32)
-        self.embedding.forward(step.tokens, resid)
+        with_step = dict(step=step) if getattr(self.embedding, "wants_step", False) else {}     # (an embedding that reads positions)
+        self.embedding.forward(step.tokens, resid, **with_step)
         if self.spec.keeps_embedding:
             step.scratch["embedding_output"] = self.embedding.forward(
-                step.tokens, rt.buffer("embedding_output", step.n_tokens, self.spec.hidden_size, torch.float32))
+                step.tokens, rt.buffer("embedding_output", step.n_tokens, self.spec.hidden_size, torch.float32), **with_step)
         stream = ResidualStream(resid, rt)
         if self._recorded_blocks is None:
             self._recorded_blocks = [self._part_replayable(b) for b in self.blocks]

@@ -19,6 +19,7 @@ import torch
 from ..config.base import ConfigError
 from ..kernels import ops
 from ..kernels import paged_attention  # noqa: F401  (registers this mixer's kernel set)
+from ..kernels import mixed_attention  # noqa: F401  (the kernel set of attention whose heads' scores are mixed)
 from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Product, TensorSpec
 
 
@@ -219,4 +220,102 @@ class NormedGQAAttention(PagedGQAAttention):
             gated = rt.buffer("nattn_gated", n, H * Dv)
             ops.heads_gate(out, P, proj if self.gate is not None else None, self.gate_col, self.gate, gated, H)
             out = gated
+        return Product(out, self.w_o)
+
+
+@MIXERS.register("mixed_heads_attention")
+class MixedHeadsAttention(NormedGQAAttention):
+    """Grouped-query attention over the paged cache whose scores pass three more steps before the softmax
+    weights exist, each a parameter:
+
+    * ``slope_exponent`` e: a distance bias, slope_g * (i - j) is taken off the score of query head g,
+      slope_g = 2^(-e (g + 1) / heads) (``None``: no bias);
+    * ``head_mix``: the heads' scores are mixed by a learned matrix, score_h <- sum_g T[h, g] score_g, after scale
+      and bias and before the window's mask and the softmax;
+    * ``sink``: a learned number per head whose exponential joins the softmax's denominator once; it has no key
+      and no value.
+
+    ``own_kv=False``: the layer has no key and value projections (nor their norm); its run-order entry reads the
+    cache of an earlier entry with equal head counts and sizes.  ``cache_window``: how many of the newest keys the
+    cache keeps (0: all); by default the mixer's own ``window``, more where another layer with a wider window
+    reads this one's cache.  Norm over the projection, value size and window are the base class's."""
+    graph_safe = True
+    lazy_input = True
+    replayable = True
+
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int | None = None,
+                 window: int = 0, scale: float | None = None, qk_norm: str | None = None, eps: float = 1e-6,
+                 slope_exponent: float | None = None, head_mix: bool = False, sink: bool = False, own_kv: bool = True,
+                 cache_window: int | None = None):
+        super().__init__(hidden_size, n_heads, n_kv_heads, head_dim, PartSpec("none", {}), value_dim=value_dim, window=window,
+                         scale=scale, qk_norm=qk_norm, eps=eps)
+        self.slope_exponent = float(slope_exponent) if slope_exponent is not None else None
+        self.head_mix, self.sink, self.own_kv = bool(head_mix), bool(sink), bool(own_kv)
+        self.cache_window = self.window if cache_window is None else int(cache_window)
+        if self.cache_window and (not self.window or self.window > self.cache_window):
+            raise ConfigError(f"mixed_heads_attention: a window of {self.window or 'all'} keys over a cache that keeps {self.cache_window}")
+        most = ops.attn_mixed_max_heads(self.stored_dim)
+        if n_heads > most:
+            raise ConfigError(f"mixed_heads_attention: {n_heads} heads of {self.stored_dim} stored values are more than the "
+                              f"kernel holds at once ({most})")
+
+    def cache_spec(self):
+        return PagedKVSpec(self.n_kv_heads, self.stored_dim, self.cache_window)
+
+    def signature_group(self):
+        return ("mixed_heads_attention", self.window)
+
+    def step_signature(self, batch):
+        return self.kernels.signature(batch, self.window)
+
+    @classmethod
+    def step_metadata_for(cls, batch, mixers):
+        return {}
+
+    def tensors(self):
+        H = self.n_heads
+        t = super().tensors()
+        if not self.own_kv:
+            for name in ("k.weight", "v.weight", "k_norm.weight"):
+                t.pop(name, None)
+        if self.head_mix:
+            eye = lambda g, shape, device: torch.eye(shape[0], device=device) + 0.3 * torch.randn(shape, generator=g, device=device)
+            t["talk"] = TensorSpec((H, H), "vector32", init=eye)
+        if self.sink:
+            t["sink"] = TensorSpec((H,), "vector32", init="normal")
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.kernels = rt.kernels("mixed_heads_attention")
+        H, G, D, Dv = self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim
+        joined = [weights["q.weight"]] + ([weights["k.weight"], weights["v.weight"]] if self.own_kv else [])
+        self.w_in = rt.prepare_weight(torch.cat(joined, dim=0).contiguous())
+        self.cols = (0, H * D, H * D + G * D) if self.own_kv else (0, -1, -1)
+        self.q_gain, self.k_gain = weights.get("q_norm.weight"), weights.get("k_norm.weight")
+        self.w_o = rt.prepare_weight(weights["o.weight"])
+        self.talk, self.sinks = weights.get("talk"), weights.get("sink")
+        self.slopes = None
+        if self.slope_exponent is not None:
+            self.slopes = torch.tensor([2.0 ** (-self.slope_exponent * (g + 1) / H) for g in range(H)], dtype=torch.float32, device=rt.device)
+        self.position.bind({}, rt)
+
+    def forward(self, x, step, cache):
+        rt, n = self.rt, x.shape[0]
+        H, D, Dv, P = self.n_heads, self.head_dim, self.value_dim, self.stored_dim
+        if cache.writes != self.own_kv:
+            raise RuntimeError("mixed_heads_attention: a layer with projections of its own writes its cache, one without reads another's")
+        table = step.block_tables[cache.group]
+        proj = rt.buffer("amix_proj", n, self.w_in.rows, torch.float32)
+        rt.gemm(x, self.w_in, proj)
+        q = rt.buffer("amix_q", n, H * P)
+        ops.qkv_prepare(proj, self.cols, step.positions, step.tok_seq, table, q, cache.kv, H, D, Dv, 0, False, None,
+                        self.q_gain, self.k_gain, self.qk_norm == "head", self.eps, write_cache=cache.writes,
+                        row_scales=rt.buffer("amix_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None)
+        out = rt.buffer("amix_out", n, H * P)
+        self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, self.slopes, self.talk, self.sinks)
+        if P != Dv:
+            packed = rt.buffer("amix_packed", n, H * Dv)
+            ops.heads_gate(out, P, None, 0, None, packed, H)
+            out = packed
         return Product(out, self.w_o)

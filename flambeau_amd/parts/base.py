@@ -284,6 +284,11 @@ class Norm(Part):
         ``store_sum`` the sum is written back to ``x``; ``rows`` selects rows."""
         raise NotImplementedError
 
+    def add_to(self, resid, delta, cast=None):
+        """Optional, for arrangements that norm a sublayer's output: ``resid += norm(delta)`` (``delta`` a float32
+        tensor); ``cast`` (or None) receives the new stream in its own dtype."""
+        raise NotImplementedError(f"{type(self).__name__} cannot norm a sublayer's output into the stream")
+
     def after_product(self, rt, resid, product: Product):
         """Optional fusion: add ``product`` to ``resid`` and return the normed sum as an object
         that ``rt.gemm`` and ``rt.gemm_swiglu`` take in place of a tensor, or ``None`` if this

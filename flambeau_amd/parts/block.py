@@ -16,6 +16,7 @@ class ResidualStream:
         self.resid = resid          # float32 [n, hidden]
         self.rt = rt
         self.pending = None         # float32 [n, hidden] not yet added, or a Product not yet computed
+        self.cast = None            # the stream in the compute dtype, where a kernel left it beside the float one
 
     def push(self, delta):
         """``delta``: what a part returned, a tensor or a ``Product``."""
@@ -31,7 +32,28 @@ class ResidualStream:
         if self._pending_tensor() is not None:
             ops.add_inplace(self.resid, self.pending)
             self.pending = None
+            self.cast = None
         return self.resid
+
+    def values(self, name="stream_values"):
+        """The stream itself (no norm) as a sublayer's input: in the compute dtype, pending sums added."""
+        resid = self.flush()
+        if resid.dtype == self.rt.dtype:
+            return resid
+        if self.cast is None:
+            self.cast = ops.cast_rows(resid, self.rt.buffer(name, resid.shape[0], resid.shape[1]))
+        return self.cast
+
+    def add_normed(self, norm, delta, name="stream_values"):
+        """``stream += norm(delta)``: the norm stands behind the sublayer.  ``delta``: what a part returned, a
+        tensor or a ``Product``.  The kernel leaves the new stream in the compute dtype too, for the sublayer
+        that reads it next."""
+        resid = self.flush()
+        if isinstance(delta, Product):
+            delta = delta.compute(self.rt)
+        cast = None if resid.dtype == self.rt.dtype else self.rt.buffer(name, resid.shape[0], resid.shape[1])
+        norm.add_to(resid, delta, cast=cast)
+        self.cast = cast
 
     def normed(self, norm, rows=None, name="normed", lazy=False):
         """The normed stream in the compute dtype, the pending delta added on the way.  With
@@ -89,6 +111,19 @@ class PreNormBlock(Block):
         stream.push(self.mixer.forward(stream.normed(self.mixer_norm, lazy=self.mixer.lazy_input), step, cache))
         if self.ffn is not None:
             stream.push(self.ffn.forward(stream.normed(self.ffn_norm, lazy=self.ffn.lazy_input), step))
+
+
+@BLOCKS.register("outnorm")
+class OutputNormBlock(PreNormBlock):
+    """Norm on the sublayer's output only: x += Norm1(Mixer(x)); x += Norm2(FeedForward(x)).  The sublayers read
+    the stream itself.  ``feed_forward`` may be ``None`` (then there is no second norm).  The norm must offer
+    ``add_to``."""
+    replayable = True
+
+    def forward(self, stream, step, cache):
+        stream.add_normed(self.mixer_norm, self.mixer.forward(stream.values(), step, cache))
+        if self.ffn is not None:
+            stream.add_normed(self.ffn_norm, self.ffn.forward(stream.values(), step))
 
 
 @BLOCKS.register("parallel")

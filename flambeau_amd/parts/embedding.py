@@ -13,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import EMBEDDINGS, HEADS, Part, TensorSpec
+from .base import EMBEDDINGS, HEADS, NORMS, Part, TensorSpec
 
 
 @EMBEDDINGS.register("token_embedding")
@@ -71,3 +71,52 @@ class ScaledTokenEmbedding(TokenEmbedding):
 
     def forward(self, tokens, out):
         return ops.embed_scaled(self.weight, tokens, out, self.scale)
+
+
+@EMBEDDINGS.register("positional_token_embedding")
+class PositionalTokenEmbedding(TokenEmbedding):
+    """h0[i, :] = E[token[i], :] + P[position[i], :] (a learned row per position, not scaled), then an optional
+    norm (any registered one).  ``wants_step``: ``forward`` is given the step, whose positions it reads."""
+    wants_step = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, max_positions: int, norm=None):
+        super().__init__(vocab_size, hidden_size)
+        self.max_positions = max_positions
+        self.norm = NORMS.create(norm) if norm is not None else None
+
+    def subparts(self):
+        return [self.norm] if self.norm is not None else []
+
+    def tensors(self):
+        t = {"weight": TensorSpec((self.vocab_size, self.hidden_size), "table"),
+             "positions": TensorSpec((self.max_positions, self.hidden_size), "table")}
+        if self.norm is not None:
+            t.update({"norm." + k: v for k, v in self.norm.tensors().items()})
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.weight, self.positions = weights["weight"], weights["positions"]
+        if self.norm is not None:
+            self.norm.bind({k[5:]: v for k, v in weights.items() if k.startswith("norm.")}, rt)
+
+    def forward(self, tokens, out, step=None):
+        if step is None:
+            raise RuntimeError("positional_token_embedding: the step (its positions) is needed")
+        ops.embed_positions(self.weight, self.positions, tokens, step.positions, out)
+        if self.norm is not None:
+            self.norm.forward(out, out)
+        return out
+
+
+@HEADS.register("scaled_linear_head")
+class ScaledOutputHead(OutputHead):
+    """logits = (x W^T) * scale, the factor applied to the 32-bit products."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float, tied: bool = False):
+        super().__init__(vocab_size, hidden_size, tied)
+        self.scale = float(scale)
+
+    def forward(self, x, max_rows):
+        logits = super().forward(x, max_rows)
+        return ops.scale_inplace(logits, self.scale) if self.scale != 1.0 else logits

@@ -13,6 +13,11 @@ per (token, head) a decay g = exp(-exp(A_log) softplus(W_a h + dt_bias)) and a w
 beta = sigmoid(W_b h); u = beta (v - S^T k) with the decayed S: the memory is corrected towards v at
 the key, not just added to.  Query/key head of head h: h // (heads / qk_heads).  Every head's o is
 divided by its root mean square, times a gain shared by the heads, times silu of a projection.
+
+HGRN2: the forget gate is a vector per head (one value per key dim) and also decides what is written:
+S <- diag(f) S + (1 - f) v^T, o = S^T q, with f = l + (1 - l) sigmoid(W_f h + b_f) above a learned lower bound
+l, q = silu(W_q h), no key of its own and no other scale.  Every head's o is divided by its root mean square
+and multiplied by a gain shared by the heads.
 """
 from __future__ import annotations
 
@@ -162,4 +167,62 @@ class GatedDelta(Mixer):
                         step.seq_q_len, step.seq_slots, hidden, H, G, D, Dv, token_gates=gates)
         out = rt.buffer("gd_out", n, H * Dv)
         ops.headnorm_gate(hidden, self.norm, proj, self.col_g, out, H, self.eps, gate_kind="silu")
+        return Product(out, self.w_o)
+
+
+@MIXERS.register("hgrn2")
+class Hgrn2(Mixer):
+    graph_safe = False          # a step run twice advances the state twice
+    replayable = True
+    lazy_input = True           # its input goes to the joined projection only
+
+    def __init__(self, hidden_size: int, n_heads: int, head_dim: int, value_dim: int, eps: float, lower_bound: bool = True,
+                 gate_bias: bool = True):
+        if head_dim > ops.linear_scan_max_dim():
+            raise ConfigError(f"hgrn2: 'dim' {head_dim} is beyond what the kernel takes ({ops.linear_scan_max_dim()})")
+        self.hidden_size, self.n_heads, self.head_dim, self.value_dim = hidden_size, n_heads, head_dim, value_dim
+        self.eps = float(eps)
+        self.lower_bound, self.gate_bias = bool(lower_bound), bool(gate_bias)
+
+    def cache_spec(self):
+        return StateSpec((self.n_heads * self.head_dim * self.value_dim,), torch.float32)
+
+    def signature_group(self):
+        return ("hgrn2",)
+
+    def step_signature(self, batch):
+        return ()
+
+    def tensors(self):
+        W, H, D, Dv = self.hidden_size, self.n_heads, self.head_dim, self.value_dim
+        t = {"q.weight": TensorSpec((H * D, W)), "f.weight": TensorSpec((H * D, W)), "v.weight": TensorSpec((H * Dv, W)),
+             "norm.weight": TensorSpec((Dv,), "vector32"), "o.weight": TensorSpec((W, H * Dv))}
+        if self.gate_bias:
+            t["f.bias"] = TensorSpec((H * D,), "vector32", init="normal")
+        if self.lower_bound:
+            t["lower"] = TensorSpec((H * D,), "vector32", init=lambda g, shape, device: torch.rand(shape, generator=g, device=device))
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        H, D, Dv = self.n_heads, self.head_dim, self.value_dim
+        self.w_in = rt.prepare_weight(torch.cat([weights["q.weight"], weights["f.weight"], weights["v.weight"]], dim=0).contiguous())
+        self.col_f, self.col_v = H * D, 2 * H * D
+        self.f_bias, self.lower = weights.get("f.bias"), weights.get("lower")
+        self.norm = weights["norm.weight"].repeat(H).contiguous()          # one gain for every head, laid out heads x vdim
+        self.w_o = rt.prepare_weight(weights["o.weight"])
+
+    def forward(self, x, step, cache):
+        rt, n = self.rt, x.shape[0]
+        H, D, Dv = self.n_heads, self.head_dim, self.value_dim
+        proj = rt.buffer("hgrn_proj", n, self.w_in.rows, torch.float32)
+        rt.gemm(x, self.w_in, proj)
+        q = rt.buffer("hgrn_q", n, H * D, torch.float32)
+        f = rt.buffer("hgrn_f", n, H * D, torch.float32)
+        ops.forget_gates(proj, 0, self.col_f, self.f_bias, self.lower, q, f)
+        hidden = rt.buffer("hgrn_hidden", n, H * Dv, torch.float32)
+        ops.linear_scan(q, f, proj[:, self.col_v:self.col_v + H * Dv], cache.state, step.seq_q_start, step.seq_q_len,
+                        step.seq_slots, hidden, H, H, D, Dv, channel_decay=True)
+        out = rt.buffer("hgrn_out", n, H * Dv)
+        ops.headnorm_gate(hidden, self.norm, None, 0, out, H, self.eps)
         return Product(out, self.w_o)

@@ -22,30 +22,40 @@ from .base import FEED_FORWARDS, FeedForward, Product, TensorSpec
 
 @FEED_FORWARDS.register("mlp")
 class Mlp(FeedForward):
-    """d = W_down act(W_up h); ``activation``: ``gelu`` (error function), ``gelu_tanh`` or ``silu``."""
+    """d = W_down act(W_up h (+ b_up)) (+ b_down); ``activation``: ``gelu`` (error function), ``gelu_tanh``, ``silu``
+    or ``relu2`` (the square of relu); ``bias``: both products have one."""
     replayable = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu"):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu", bias: bool = False):
         if activation not in ops.ACTIVATIONS:
             raise ValueError(f"mlp: unknown activation '{activation}'; known: {sorted(ops.ACTIVATIONS)}")
         self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+        self.has_bias = bool(bias)
 
     def tensors(self):
         W, F = self.hidden_size, self.intermediate_size
-        return {"up.weight": TensorSpec((F, W)), "down.weight": TensorSpec((W, F))}
+        t = {"up.weight": TensorSpec((F, W)), "down.weight": TensorSpec((W, F))}
+        if self.has_bias:
+            t.update({"up.bias": TensorSpec((F,), "vector32", init="normal"), "down.bias": TensorSpec((W,), "vector32", init="normal")})
+        return t
 
     def bind(self, weights, rt):
         self.rt = rt
         self.w_up = rt.prepare_weight(weights["up.weight"])
         self.w_down = rt.prepare_weight(weights["down.weight"])
+        self.b_up, self.b_down = weights.get("up.bias"), weights.get("down.bias")
 
     def forward(self, x, step):
         rt, n, F = self.rt, x.shape[0], self.intermediate_size
         pre = rt.buffer("mlp_pre", n, F, torch.float32)
         rt.gemm(x, self.w_up, pre)
         act = rt.buffer("mlp_act", n, F)
-        ops.activation(pre, act, self.activation)
-        return Product(act, self.w_down)
+        ops.activation(pre, act, self.activation, bias=self.b_up)
+        if self.b_down is None:
+            return Product(act, self.w_down)
+        delta = rt.buffer("mlp_delta", n, self.hidden_size, torch.float32)
+        rt.gemm(act, self.w_down, delta)
+        return ops.add_rowvec(delta, self.b_down)
 
 
 @FEED_FORWARDS.register("routed_experts")
@@ -53,11 +63,20 @@ class RoutedExperts(FeedForward):
     replayable = True
 
     def __init__(self, hidden_size: int, n_experts: int, top: int, expert_size: int, shared_size: int | None = None,
-                 scoring: str = "sigmoid", renormalise: bool = False, weight_on: str = "input", shared_gate: bool = True):
+                 scoring: str = "sigmoid", renormalise: bool = False, weight_on: str = "input", shared_gate: bool = True,
+                 gated: bool = True, activation: str = "silu", router_bias: bool = False):
+        """``scoring``: ``sigmoid``, ``softmax`` (over all experts) or ``softmax_chosen`` (over the chosen logits only);
+        ``gated=False``: an expert is W_down act(W_up u) with ``activation`` (no gate matrix); ``router_bias``: the
+        router's logits have a bias."""
         if weight_on not in ("input", "output"):
             raise ValueError(f"routed_experts: weight_on must be 'input' or 'output', got {weight_on!r}")
-        if scoring not in ("sigmoid", "softmax"):
-            raise ValueError(f"routed_experts: scoring must be 'sigmoid' or 'softmax', got {scoring!r}")
+        if scoring not in ops.ROUTER_SCORINGS:
+            raise ValueError(f"routed_experts: scoring must be one of {sorted(ops.ROUTER_SCORINGS)}, got {scoring!r}")
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"routed_experts: unknown activation '{activation}'; known: {sorted(ops.ACTIVATIONS)}")
+        if gated and activation != "silu":
+            raise ValueError("routed_experts: gated experts take the silu gate")
+        self.gated, self.activation, self.router_bias = bool(gated), activation, bool(router_bias)
         self.hidden_size, self.n_experts, self.top = hidden_size, n_experts, top
         self.expert_size, self.shared_size = expert_size, shared_size
         self.scoring, self.renormalise, self.weight_on = scoring, bool(renormalise), weight_on
@@ -66,8 +85,11 @@ class RoutedExperts(FeedForward):
     def tensors(self):
         W, F = self.hidden_size, self.expert_size
         t = {"router.weight": TensorSpec((self.n_experts, W))}
+        if self.router_bias:
+            t["router.bias"] = TensorSpec((self.n_experts,), "vector32", init="normal")
         for e in range(self.n_experts):
-            t[f"e{e}.gate.weight"] = TensorSpec((F, W))
+            if self.gated:
+                t[f"e{e}.gate.weight"] = TensorSpec((F, W))
             t[f"e{e}.up.weight"] = TensorSpec((F, W))
             t[f"e{e}.down.weight"] = TensorSpec((W, F))
         if self.shared_size is not None:
@@ -84,7 +106,12 @@ class RoutedExperts(FeedForward):
         # the router's rows and, behind them, the shared expert's gate: one plain product gives all logits
         rows = [weights["router.weight"]] + ([weights["shared.sg.weight"]] if self.shared_gate else [])
         self.w_logits = torch.cat(rows, dim=0).contiguous()
-        self.w_gate_up = torch.stack([torch.cat([weights[f"e{e}.gate.weight"], weights[f"e{e}.up.weight"]], dim=0) for e in range(E)]).contiguous()
+        first = (lambda e: torch.cat([weights[f"e{e}.gate.weight"], weights[f"e{e}.up.weight"]], dim=0)) if self.gated else (lambda e: weights[f"e{e}.up.weight"])
+        self.w_gate_up = torch.stack([first(e) for e in range(E)]).contiguous()       # (ungated experts: the up matrices alone)
+        self.b_logits = None
+        if self.router_bias:
+            extra = self.w_logits.shape[0] - E
+            self.b_logits = torch.cat([weights["router.bias"], torch.zeros(extra, dtype=torch.float32, device=weights["router.bias"].device)]).contiguous()
         self.w_down = torch.stack([weights[f"e{e}.down.weight"] for e in range(E)]).contiguous()
         if self.shared_size is not None:
             self.ws_gate_up = rt.prepare_gate_up(weights["shared.gate.weight"], weights["shared.up.weight"])
@@ -97,6 +124,8 @@ class RoutedExperts(FeedForward):
         most = rt.max_batch_tokens * top
         logits = rt.buffer("moe_logits", n, self.w_logits.shape[0], torch.float32)
         ops.gemm_few(x, self.w_logits, logits)
+        if self.b_logits is not None:
+            ops.add_rowvec(logits, self.b_logits)
         ints = lambda name, rows, cols, cap: rt.buffer(name, rows, cols, torch.int32, max_rows=cap)
         place = ints("moe_place", pairs, 1, most).view(-1)
         src_row = ints("moe_src_row", pairs, 1, most).view(-1)
@@ -106,10 +135,13 @@ class RoutedExperts(FeedForward):
         tiles = ints("moe_tiles", n_tiles, 4, ops.moe_max_tiles(most, E))
         ops.moe_route(logits, 0, E, top, place, src_row, src_scale, pair_w, tiles, self.scoring, self.renormalise)
         on_input = self.weight_on == "input"
-        gate_up = rt.buffer("moe_gate_up", pairs, 2 * F, torch.float32, max_rows=most)
+        gate_up = rt.buffer("moe_gate_up", pairs, (2 if self.gated else 1) * F, torch.float32, max_rows=most)
         ops.moe_gemm(x, self.w_gate_up, gate_up, tiles, src_row, src_scale if on_input else None, matrix_cores=rt.tuned)
         act = rt.buffer("moe_act", pairs, F, max_rows=most)
-        ops.silu_mul(gate_up, act)
+        if self.gated:
+            ops.silu_mul(gate_up, act)
+        else:
+            ops.activation(gate_up, act, self.activation)
         y = rt.buffer("moe_y", pairs, W, torch.float32, max_rows=most)
         ops.moe_gemm(act, self.w_down, y, tiles, None, None if on_input else src_scale, matrix_cores=rt.tuned)
         shared = None

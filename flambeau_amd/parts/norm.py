@@ -66,3 +66,33 @@ class DynamicTanh(Norm):
         sum in its epilogue (nothing crosses the values of a row, so the norm is finished there): the normed
         rows come back as a tensor and no norm kernel runs."""
         return rt.gemm_add_dyt(product.x, product.weight, resid, self.alpha, self.weight, self.bias)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Norm):
+    """y = (x - mean) / sqrt(var + eps) * w + b over a row, var the mean of the squared deviations;
+    ``bias=False`` leaves b out.  Beside ``forward`` it offers ``add_to``: the norm of a sublayer's OUTPUT
+    added to the stream, for arrangements that norm what a sublayer returns and not what it reads."""
+    replayable = True
+
+    def __init__(self, hidden_size: int, eps: float, bias: bool = True):
+        self.hidden_size = hidden_size
+        self.eps = float(eps)
+        self.has_bias = bool(bias)
+
+    def tensors(self):
+        t = {"weight": TensorSpec((self.hidden_size,), "vector32")}
+        if self.has_bias:
+            t["bias"] = TensorSpec((self.hidden_size,), "vector32", init="normal")
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.weight, self.bias = weights["weight"], weights.get("bias")
+
+    def forward(self, x, out, delta=None, store_sum=False, rows=None):
+        return ops.layernorm(x, self.weight, self.bias, out, self.eps, delta=delta, store_sum=store_sum, rows=rows)
+
+    def add_to(self, resid, delta, cast=None):
+        """``resid += norm(delta)``; ``cast`` (a tensor of the compute dtype, or None) receives the new stream."""
+        return ops.layernorm_add(delta, self.weight, self.bias, resid, self.eps, cast=cast)
