@@ -25,6 +25,10 @@ JSON line; ``value`` is Kuvidra's decode tokens/s at the larger size, the rest i
 ``--config bugidra``: the Bugidra design (attention with normed, capped and gated extras, attention and retention side
 by side, the gated delta rule behind short convolutions, Dynamic Tanh norms) at two sizes that resemble real layers,
 beside a Mistral of the same width, head count and number of layers, measured the same way; a line of the same shape.
+
+``--config fitevik``: the Fitevik design (layer norms behind the sublayers, learned positions, the HGRN2 recurrence,
+attention inside a window with a distance bias, mixed heads and a sink, one layer reading another's keys, dense and
+routed feed-forwards with the squared relu) at two sizes, six layers, beside the same Mistral; a line of the same shape.
 """
 from __future__ import annotations
 
@@ -395,6 +399,29 @@ BUGIDRA_SIZES = {
 }
 
 
+def fitevik_config(width, heads, kv_heads, ff, experts, top, expert_ff, rec_heads, window, vocab=32768):
+    rec = {"type": "hgrn2", "mixer": dict(heads=rec_heads, dim=128, vdim=128)}
+    att = dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, mask={"size": window})
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}}
+    layers = [dict(rec, mlp=dense), dict(rec, mlp=moe), {"type": "attention", "mixer": att, "mlp": dense},
+              {"type": "attention", "mixer": dict(att, kv_from=2), "mlp": moe}, dict(rec, mlp=dense),
+              {"type": "attention", "mixer": att, "mlp": moe}]
+    return {"architecture": "Fitevik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "max_positions": 8192, "logit_scale": 0.5,
+            "layers": layers}
+
+
+FITEVIK_SIZES = {
+    "w2048": dict(width=2048, heads=16, kv_heads=8, ff=8192, experts=16, top=2, expert_ff=1024, rec_heads=16, window=1024),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, ff=14336, experts=32, top=4, expert_ff=1536, rec_heads=32, window=1024),
+}
+
+
+def bench_fitevik(a, dtype_name):
+    """The same for the Fitevik design: three recurrent and three attention layers (one reads another's keys)."""
+    return bench_design(a, dtype_name, "fitevik", "Fitevik", FITEVIK_SIZES, fitevik_config, "6 layers")
+
+
 def bench_kuvidra(a, dtype_name):
     """Prefill and decode of the Kuvidra design at layer sizes of real models, beside the closest model the engine
     has (Mistral) at the same width, head count and number of layer runs."""
@@ -452,10 +479,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--reps", type=int, default=REPS, help="repetitions of the timed steps; the median is reported")
-    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra", "bugidra"])
-    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra / bugidra: one size only")
-    ap.add_argument("--only-model", default=None, choices=["kuvidra", "bugidra", "mistral"],
-                    help="--config kuvidra / bugidra: one of the two models only")
+    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra", "bugidra", "fitevik"])
+    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra / bugidra / fitevik: one size only")
+    ap.add_argument("--only-model", default=None, choices=["kuvidra", "bugidra", "fitevik", "mistral"],
+                    help="--config kuvidra / bugidra / fitevik: one of the two models only")
     ap.add_argument("--layers", type=int, default=None, help="run only the first layers (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -474,6 +501,8 @@ def main():
         return bench_kuvidra(a, dtype_name)
     if a.config == "bugidra":
         return bench_bugidra(a, dtype_name)
+    if a.config == "fitevik":
+        return bench_fitevik(a, dtype_name)
     label, cfg = CONFIGS[a.config]
     if a.config != "7b":
         return bench_serving(a, a.config, label, cfg, dtype_name, el)

@@ -70,6 +70,19 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
         k1 = min(p, (part + 1) * a.part_keys - 1);
     }
     const int group = nh / cache.n_kv_heads;
+    {
+        // a padding row of a fixed-size batch has no page, not even for its own position: zeros, and no key is read
+        const int own = table[p / ps];
+        if (own < 0 || own >= cache.n_pages) {
+            if (a.part_keys > 0) {
+                float* pm = a.part_ml + ((size_t)token * a.n_parts + blockIdx.y) * nh * 2;
+                for (int h = tid; h < nh; h += AM_THREADS) { pm[2 * h] = -INFINITY; pm[2 * h + 1] = 0.f; }
+            } else {
+                for (int o = tid; o < nh * hd; o += AM_THREADS) out[(size_t)token * nh * hd + o] = from_f32<T>(0.f);
+            }
+            return;
+        }
+    }
     for (int e = tid; e < nh * hd; e += AM_THREADS) qs[e] = to_f32(q[(size_t)token * nh * hd + e]);
     for (int e = tid; e < nh * nh; e += AM_THREADS) tk[e] = a.talk ? a.talk[e] : 0.f;
     for (int e = tid; e < nh; e += AM_THREADS) {
@@ -88,7 +101,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
             const int g = e / AM_CHUNK, j = base + (e % AM_CHUNK);
             float s = 0.f;
             if (j >= k0 && j <= k1) {
-                const int page = table[j / ps];
+                const int page = min(max(table[j / ps], 0), cache.n_pages - 1);      // (a key inside the window always has a page)
                 const T* kr = base_ptr + cache_k_offset(cache, page, g / group, j % ps, 0);
                 const float* qg = qs + g * hd;
                 float s0 = 0.f, s1 = 0.f;
@@ -150,7 +163,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
                 for (int j8 = 0; j8 < AM_CHUNK; j8 += 8) {
                     const int j = base + j8;
                     if (j + 7 < k0 || j > k1) continue;
-                    const int page = table[j / ps];
+                    const int page = min(max(table[j / ps], 0), cache.n_pages - 1);
                     Vec8<T> vv;
                     vv.load(base_ptr + cache_v_offset(cache, page, h / group, j % ps, d));
 #pragma unroll
@@ -164,7 +177,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
                     const int j = base + jj;
                     const float w = ph[jj];
                     if (j < k0 || j > k1 || w == 0.f) continue;
-                    sum = fmaf(w, to_f32(base_ptr[cache_v_offset(cache, table[j / ps], h / group, j % ps, d)]), sum);
+                    sum = fmaf(w, to_f32(base_ptr[cache_v_offset(cache, min(max(table[j / ps], 0), cache.n_pages - 1), h / group, j % ps, d)]), sum);
                 }
             }
             acc[u] = sum;

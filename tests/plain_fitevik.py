@@ -84,29 +84,39 @@ def keys_and_values(h, m, t, p, eps):
     return k, v
 
 
+def mixed_softmax_attention(q, k, v, window, scale, slopes, talk, sink, first=0):
+    """``q`` [T, H, dim] at positions first .. first + T - 1; ``k`` [first + T, G, dim] and ``v`` [first + T, G, vdim]
+    from position 0.  raw_g = scale q_g . k_j - slope_g (i - j); score_h = sum_g talk[h, g] raw_g; inside the
+    window softmax with exp(sink_h) added to the denominator.  ``slopes``, ``talk``, ``sink`` may be None."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    kv_of = [g // (H // G) for g in range(H)]
+    out = np.zeros((T, H, v.shape[2]))
+    for r in range(T):
+        i = first + r
+        lo = max(0, i - window + 1) if window else 0
+        raw = np.zeros((H, i + 1 - lo))
+        for g in range(H):
+            raw[g] = k[lo:i + 1, kv_of[g]] @ q[r, g] * scale
+            if slopes is not None:
+                raw[g] -= slopes[g] * (i - np.arange(lo, i + 1))
+        mixed = talk @ raw if talk is not None else raw                      # [H, keys]
+        for g in range(H):
+            top = mixed[g].max() if sink is None else max(mixed[g].max(), sink[g])
+            e = np.exp(mixed[g] - top)
+            w = e / (e.sum() + (math.exp(sink[g] - top) if sink is not None else 0.0))   # the sink counts once and has no value
+            out[r, g] = w @ v[lo:i + 1, kv_of[g]]
+    return out
+
+
 def attention(h, m, t, p, eps, k, v):
     """Softmax attention inside a sliding window with a distance bias, scores mixed over the heads, and a
     sink in the denominator.  ``k`` [T, G, dim], ``v`` [T, G, vdim]: this layer's or another's."""
     T = h.shape[0]
-    H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    window, scale = m["mask"]["size"], m["scale"]
+    H, D = m["heads"], m["dim"]
     q = rms_norm(h @ t[p + "q"].T, t[p + "q.norm"], eps).reshape(T, H, D)
-    kv_of = [g // (H // G) for g in range(H)]
-    slopes = head_slopes(H)
-    talk, sink = t[p + "talk"], t[p + "sink"]
-    out = np.zeros((T, H, Dv))
-    for i in range(T):
-        lo = max(0, i - window + 1)
-        raw = np.zeros((H, i + 1 - lo))
-        for g in range(H):
-            raw[g] = k[lo:i + 1, kv_of[g]] @ q[i, g] * scale - slopes[g] * (i - np.arange(lo, i + 1))
-        mixed = talk @ raw                                                    # [H, keys]
-        for g in range(H):
-            top = max(mixed[g].max(), sink[g])
-            e = np.exp(mixed[g] - top)
-            w = e / (e.sum() + math.exp(sink[g] - top))                       # the sink counts once and has no value
-            out[i, g] = w @ v[lo:i + 1, kv_of[g]]
-    return out.reshape(T, H * Dv) @ t[p + "o"].T
+    out = mixed_softmax_attention(q, k, v, m["mask"]["size"], m["scale"], head_slopes(H), t[p + "talk"], t[p + "sink"])
+    return out.reshape(T, -1) @ t[p + "o"].T
 
 
 # ---------------------------------------------------------------- feed-forwards
@@ -155,5 +165,5 @@ def forward(cfg, t, tokens, keep_layers=False):
         if layer.get("mlp") is not None:
             x = x + layer_norm(feed_forward(x, layer["mlp"], t, p + "mlp."), t, p + "norm2", eps)
         streams.append(x.copy())
-    logits = output(x, t, eps, cfg["logit_scale"])
+    logits = output(x, t, eps, cfg.get("logit_scale", 1.0))
     return (logits, np.stack(streams)) if keep_layers else logits
