@@ -356,9 +356,10 @@ def test_single_tokens_behind_a_long_window_deal_their_keys_out():
         x = _x(n, W, "bfloat16", 5)
         want = plain_mixed(x.double().numpy(), plain, H, G, D, Dv, window, 0.5, eps, first=n - 20)
         seen = []
-        orig = mixer.kernels.signature
-        mixer.kernels.signature = lambda batch, w: seen.append(orig(batch, w)) or seen[-1]
+        orig = type(mixer.kernels).signature
+        mixer.kernels.signature = lambda batch, w, k=mixer.kernels: seen.append(orig(k, batch, w)) or seen[-1]
         got = run_mixer(mixer, rt, x, [n - 20, 3] + [1] * 17, page_size=16, n_pages=64)
+        del mixer.kernels.signature
         assert max(seen) >= 4 and seen[0] == 0               # the prompt: a block per token; the single tokens: parts
         assert np.abs(got[n - 20:] - want).max() < 3e-2 * np.abs(want).max(), window
 
