@@ -345,6 +345,12 @@ int fl_attn_mixed(const void* q, void* out, const void* cache_base, int dtype, c
                   int page_size, int n_pages, float scale, int window, const float* slopes, const float* talk,
                   const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
                   hipStream_t stream);
+int fl_attn_mixed_tiled_fits(int nh, int hd, int page_size);
+int fl_attn_mixed_tiled(const void* q, void* out, const void* cache_base, const int* positions, const int* block_table,
+                        int max_blocks, const int* seq_q_start, const int* seq_q_len, int n_seqs, int n_tiles, int n,
+                        int nh, int nkv, int hd, int page_size, int n_pages, float scale, int window, const float* slopes,
+                        const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
+                        hipStream_t stream);
 
 // ---- step programs (program.hip): launches recorded once, replayed with one call ----
 typedef union FlArg { void* p; long l; int i; float f; } FlArg;

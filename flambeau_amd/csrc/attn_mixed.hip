@@ -212,25 +212,25 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
     }
 }
 
-// joins the parts of a token (rising order) and adds the sink: a thread per (token, head, dim)
+// joins the parts of a token (rising order) and adds the sink: a block per (token, head), a thread per dim
 template <typename T>
-__global__ __launch_bounds__(AM_THREADS) void attn_mixed_join_kernel(T* __restrict__ out, AttnMixed a, int hd) {
-    const int token = blockIdx.x, nh = a.nh;
-    for (int o = threadIdx.x; o < nh * hd; o += AM_THREADS) {
-        const int h = o / hd;
-        const float* pm = a.part_ml + (size_t)token * a.n_parts * nh * 2;
-        const float sk = a.sink ? a.sink[h] : -INFINITY;
-        float top = sk;
-        for (int part = 0; part < a.n_parts; ++part) top = fmaxf(top, pm[(part * nh + h) * 2]);
+__global__ __launch_bounds__(128) void attn_mixed_join_kernel(T* __restrict__ out, AttnMixed a, int hd) {
+    const int token = blockIdx.x, h = blockIdx.y, nh = a.nh;
+    const float* pm = a.part_ml + (size_t)token * a.n_parts * nh * 2;
+    const float sk = a.sink ? a.sink[h] : -INFINITY;
+    float top = sk;
+    for (int part = 0; part < a.n_parts; ++part)
+        if (pm[(part * nh + h) * 2 + 1] > 0.f) top = fmaxf(top, pm[(part * nh + h) * 2]);
+    for (int d = threadIdx.x; d < hd; d += 128) {
         float den = a.sink ? expf(sk - top) : 0.f, num = 0.f;
         for (int part = 0; part < a.n_parts; ++part) {
             const float m = pm[(part * nh + h) * 2], l = pm[(part * nh + h) * 2 + 1];
             if (!(l > 0.f)) continue;                                         // a part without keys
             const float f = expf(m - top);
             den = fmaf(l, f, den);
-            num = fmaf(a.part_acc[((size_t)token * a.n_parts + part) * nh * hd + o], f, num);
+            num = fmaf(a.part_acc[(((size_t)token * a.n_parts + part) * nh + h) * hd + d], f, num);
         }
-        out[(size_t)token * nh * hd + o] = from_f32<T>(den > 0.f ? num / den : 0.f);
+        out[((size_t)token * nh + h) * hd + d] = from_f32<T>(den > 0.f ? num / den : 0.f);
     }
 }
 
@@ -274,8 +274,8 @@ extern "C" int fl_attn_mixed(const void* q, void* out, const void* cache_base, i
     else FL_CHECK(false, "attn_mixed: unknown dtype %d", dtype);
     FL_LAUNCH_CHECK();
     if (part_keys > 0) {
-        if (dtype == FL_F32) attn_mixed_join_kernel<float><<<n, AM_THREADS, 0, stream>>>((float*)out, a, hd);
-        else attn_mixed_join_kernel<bf16_t><<<n, AM_THREADS, 0, stream>>>((bf16_t*)out, a, hd);
+        if (dtype == FL_F32) attn_mixed_join_kernel<float><<<dim3(n, nh), 128, 0, stream>>>((float*)out, a, hd);
+        else attn_mixed_join_kernel<bf16_t><<<dim3(n, nh), 128, 0, stream>>>((bf16_t*)out, a, hd);
         FL_LAUNCH_CHECK();
     }
 #undef FL_AM_T
@@ -283,3 +283,299 @@ extern "C" int fl_attn_mixed(const void* q, void* out, const void* cache_base, i
     return 0;
 }
 FL_RECORDABLE(fl_attn_mixed)
+
+
+// ---------------------------------------------------------------------------------------------------------
+// The same attention on the matrix cores, for bfloat16 caches: a block of eight waves takes up to 16
+// consecutive query tokens of one request with ALL heads and walks their keys in chunks of 32 (aligned to
+// absolute positions).  Per chunk, with a barrier between the phases:
+//   1. raw[g][query][key] = scale * Q_g . K^T - slope_g * (i - j)      v_mfma_f32_16x16x32_bf16, float into LDS;
+//      the (head, half chunk) tiles are dealt out to the waves, operands come straight from q and the pages
+//   2. score[h][pair] = sum_g talk[h][g] * raw[g][pair]                v_mfma_f32_16x16x4_f32 (true 32-bit): the
+//      mixing matrix is the A operand and lives in registers, 16 (query, key) pairs are a B operand's columns
+//   3. a thread per (head, query) row: mask, running maximum and sum (they stay in that thread's registers from
+//      chunk to chunk), weights as bfloat16 into LDS, and the factor by which the row's output shrinks
+//   4. out[h][query][:] = factor * out + P_h . V                        v_mfma_f32_16x16x32_bf16; a wave owns heads
+//      wave, wave + 8, ...; values lie transposed in a page, so eight keys of one dim are one 16-byte load
+// Which block takes which tile is found from the step's own lists (first row and rows of every request).
+// With part_keys > 0 a tile's keys are dealt out to n_parts blocks as above and joined by the same kernel.
+#define AT_ROWS 16
+#define AT_CHUNK 32
+#define AT_THREADS 512
+#define AT_WAVES 8
+#define AT_RAW_LD (AT_ROWS * AT_CHUNK + 16)     // floats per head of raw (the 16 spread the four heads of an operand over the banks)
+#define AT_SC_LD (AT_ROWS * (AT_CHUNK + 1))     // floats per head of score: rows of 33
+#define AT_P_LD 40                              // bfloat16 per row of weights
+#define AT_MAX_HEADS 32
+
+struct AttnTiles {
+    const int* seq_q_start; const int* seq_q_len; int n_seqs;
+};
+
+template <int DT>
+__global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                                                                       PagedCache cache, AttnMixed a, AttnTiles tl) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    __shared__ int s_tile[3];
+    const int nh = a.nh, hd = cache.head_dim, ps = cache.page_size;
+    const int HP = (nh + 15) & ~15;
+    float* raw = lds;                                   // [HP][AT_RAW_LD]
+    float* sc = raw + HP * AT_RAW_LD;                   // [HP][16][33]
+    float* corr = sc + HP * AT_SC_LD;                   // [HP][16]
+    bf16_t* pb = (bf16_t*)raw;                          // [nh][16][AT_P_LD]: the weights take raw's place once it is mixed
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+
+    // ---- which rows: tile blockIdx.x of the requests' portions, 16 rows each
+    if (tid == 0) {
+        int t = blockIdx.x, seq = -1, row0 = 0, cnt = 0;
+        for (int s = 0; s < tl.n_seqs; ++s) {
+            const int len = tl.seq_q_len[s], nt = (len + AT_ROWS - 1) / AT_ROWS;
+            if (t < nt) { seq = s; row0 = tl.seq_q_start[s] + AT_ROWS * t; cnt = min(AT_ROWS, len - AT_ROWS * t); break; }
+            t -= nt;
+        }
+        s_tile[0] = seq; s_tile[1] = row0; s_tile[2] = cnt;
+    }
+    __syncthreads();
+    const int seq = s_tile[0], row0 = s_tile[1], cnt = s_tile[2];
+    if (seq < 0) return;
+    const int p_first = a.positions[row0], p_last = p_first + cnt - 1;
+    const int* table = a.block_table + (size_t)seq * a.max_blocks;
+    const int safe_page = table[p_last / ps];
+    const bool live = safe_page >= 0 && safe_page < cache.n_pages;      // (a padding row of a fixed-size batch has no page)
+    const int lo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+    int k0 = lo, k1 = p_last;
+    if (a.part_keys > 0) {
+        const int part = lo / a.part_keys + blockIdx.y;
+        k0 = max(lo, part * a.part_keys);
+        k1 = min(p_last, (part + 1) * a.part_keys - 1);
+    }
+    if (!live || k0 > k1) {
+        if (a.part_keys > 0) {
+            for (int e = tid; e < cnt * nh; e += AT_THREADS) {
+                float* pm = a.part_ml + (((size_t)(row0 + e / nh) * a.n_parts + blockIdx.y) * nh + e % nh) * 2;
+                pm[0] = -INFINITY; pm[1] = 0.f;
+            }
+        } else {
+            for (int e = tid; e < cnt * nh * hd; e += AT_THREADS) out[(size_t)row0 * nh * hd + e] = (bf16_t)0.f;
+        }
+        return;
+    }
+    const int group = nh / cache.n_kv_heads;
+    const bf16_t* kv = (const bf16_t*)cache.base;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // ---- the mixing matrix as A operands: tA[hb][kk] = talk[16 hb + li][4 kk + lg] (the unit matrix without one)
+    float tA[2][AT_MAX_HEADS / 4];
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+        for (int kk = 0; kk < AT_MAX_HEADS / 4; ++kk) {
+            const int h = 16 * hb + li, g = 4 * kk + lg;
+            tA[hb][kk] = (h < nh && g < nh) ? (a.talk ? a.talk[h * nh + g] : (h == g ? 1.f : 0.f)) : 0.f;
+        }
+    for (int e = tid; e < (HP - nh) * AT_RAW_LD; e += AT_THREADS) raw[nh * AT_RAW_LD + e] = 0.f;     // heads that do not exist
+    // ---- the row (head, query) this thread keeps the softmax of
+    const int rh = tid >> 4, rq = tid & 15;
+    const bool row_on = rh < nh && rq < cnt;
+    const int rp = p_first + rq;
+    const int r_lo = max(k0, a.window > 0 ? rp - a.window + 1 : 0), r_hi = min(k1, rp);
+    float rm = -INFINITY, rl = 0.f;
+    f32x4 o[4][DT];
+#pragma unroll
+    for (int hi = 0; hi < 4; ++hi)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[hi][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const int ksteps = (hd + 31) / 32;
+    __syncthreads();
+
+    for (int base = (k0 / AT_CHUNK) * AT_CHUNK; base <= k1; base += AT_CHUNK) {
+        // ---- 1. raw scores of every head
+        for (int item = wave; item < 2 * nh; item += AT_WAVES) {
+            const int g = item >> 1, kt = item & 1;
+            const int jpos = base + 16 * kt + li;
+            int page = jpos <= p_last ? table[jpos / ps] : safe_page;
+            if (page < 0 || page >= cache.n_pages) page = safe_page;
+            const bf16_t* krow = kv + cache_k_offset(cache, page, g / group, jpos % ps, 0);
+            const bf16_t* qrow = q + ((size_t)(row0 + li) * nh + g) * hd;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < ksteps; ++s) {
+                const int d = 32 * s + 8 * lg;
+                const bool in = d < hd;
+                const bf16x8 kf = in ? *(const bf16x8*)(krow + d) : zero8;
+                const bf16x8 qf = (in && li < cnt) ? *(const bf16x8*)(qrow + d) : zero8;
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf, kf, acc, 0, 0, 0);
+            }
+            const float slope = a.slopes ? a.slopes[g] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int qq = 4 * lg + r;
+                raw[g * AT_RAW_LD + qq * AT_CHUNK + 16 * kt + li] = acc[r] * a.scale - slope * (float)(p_first + qq - jpos);
+            }
+        }
+        __syncthreads();
+        // ---- 2. the heads' scores mixed: 16 pairs at a time, pairs of the queries that exist
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+            if (16 * hb >= HP) continue;
+            for (int pt = wave; pt < 2 * cnt; pt += AT_WAVES) {
+                f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < AT_MAX_HEADS / 4; ++kk) {
+                    if (4 * kk >= HP) continue;
+                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(tA[hb][kk], raw[(4 * kk + lg) * AT_RAW_LD + 16 * pt + li], c, 0, 0, 0);
+                }
+                const int pair = 16 * pt + li;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    sc[(16 * hb + 4 * lg + r) * AT_SC_LD + (pair >> 5) * (AT_CHUNK + 1) + (pair & 31)] = c[r];
+            }
+        }
+        __syncthreads();
+        // ---- 3. the rows' softmax
+        if (rh < nh) {
+            unsigned* prow = (unsigned*)(pb + (rh * AT_ROWS + rq) * AT_P_LD);
+            const float* srow = sc + rh * AT_SC_LD + rq * (AT_CHUNK + 1);
+            float mx = -INFINITY;
+            if (row_on)
+                for (int j = 0; j < AT_CHUNK; ++j)
+                    if (base + j >= r_lo && base + j <= r_hi) mx = fmaxf(mx, srow[j]);
+            if (mx == -INFINITY) {                                            // no key of this chunk for this row
+                for (int j2 = 0; j2 < AT_CHUNK / 2; ++j2) prow[j2] = 0u;
+                corr[rh * AT_ROWS + rq] = 1.f;
+            } else {
+                const float m_new = fmaxf(rm, mx);
+                const float cr = rm == -INFINITY ? 0.f : expf(rm - m_new);
+                float sum = 0.f;
+                for (int j = 0; j < AT_CHUNK; j += 2) {
+                    const float e0 = (base + j >= r_lo && base + j <= r_hi) ? expf(srow[j] - m_new) : 0.f;
+                    const float e1 = (base + j + 1 >= r_lo && base + j + 1 <= r_hi) ? expf(srow[j + 1] - m_new) : 0.f;
+                    sum += e0 + e1;
+                    const bf16_t b0 = (bf16_t)e0, b1 = (bf16_t)e1;
+                    prow[j >> 1] = (unsigned)__builtin_bit_cast(unsigned short, b0) | ((unsigned)__builtin_bit_cast(unsigned short, b1) << 16);
+                }
+                rl = rl * cr + sum;
+                rm = m_new;
+                corr[rh * AT_ROWS + rq] = cr;
+            }
+        }
+        __syncthreads();
+        // ---- 4. the weighted sums of the values
+#pragma unroll
+        for (int hi = 0; hi < 4; ++hi) {
+            const int h = wave + AT_WAVES * hi;
+            if (h >= nh) continue;
+            float cr[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) cr[r] = corr[h * AT_ROWS + 4 * lg + r];
+            const bf16x8 pf = *(const bf16x8*)(pb + (h * AT_ROWS + li) * AT_P_LD + 8 * lg);
+            const int jr = base + 8 * lg;                                      // this lane's run of eight keys
+            int page = jr <= p_last ? table[jr / ps] : -1;
+            const bool run_on = page >= 0 && page < cache.n_pages && jr <= k1;
+            if (!run_on) page = safe_page;
+            const bf16_t* vbase = kv + cache_v_offset(cache, page, h / group, jr % ps, 0);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = 16 * dt + li;
+                bf16x8 vf = (run_on && d < hd) ? *(const bf16x8*)(vbase + (size_t)d * ps) : zero8;
+                if (jr + 7 > k1) {                                             // keys that nobody wrote yet may hold anything
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (jr + e > k1) vf[e] = (bf16_t)0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[hi][dt][r] *= cr[r];
+                o[hi][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[hi][dt], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- the rows' maxima and sums go to the waves that hold the outputs (or to the parts' scratch)
+    float* hm = sc;
+    float* hl = sc + HP * AT_ROWS;
+    if (rh < nh) {
+        hm[rh * AT_ROWS + rq] = rm;
+        hl[rh * AT_ROWS + rq] = rl;
+        if (a.part_keys > 0 && rq < cnt) {
+            float* pm = a.part_ml + (((size_t)(row0 + rq) * a.n_parts + blockIdx.y) * nh + rh) * 2;
+            pm[0] = rm; pm[1] = rl;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int hi = 0; hi < 4; ++hi) {
+        const int h = wave + AT_WAVES * hi;
+        if (h >= nh) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int qq = 4 * lg + r;
+            if (qq >= cnt) continue;
+            float f = 1.f;
+            if (a.part_keys == 0) {
+                const float m = hm[h * AT_ROWS + qq], l = hl[h * AT_ROWS + qq];
+                const float sk = a.sink ? a.sink[h] : -INFINITY;
+                const float top = fmaxf(m, sk);
+                const float fm = expf(m - top);
+                const float den = l * fm + (a.sink ? expf(sk - top) : 0.f);
+                f = den > 0.f ? fm / den : 0.f;
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = 16 * dt + li;
+                if (d >= hd) continue;
+                if (a.part_keys > 0) a.part_acc[(((size_t)(row0 + qq) * a.n_parts + blockIdx.y) * nh + h) * hd + d] = o[hi][dt][r];
+                else out[((size_t)(row0 + qq) * nh + h) * hd + d] = (bf16_t)(o[hi][dt][r] * f);
+            }
+        }
+    }
+}
+
+extern "C" int fl_attn_mixed_tiled_fits(int nh, int hd, int page_size) {
+    return nh >= 1 && nh <= AT_MAX_HEADS && hd % 8 == 0 && hd <= 128 && page_size % 8 == 0;
+}
+
+// ``n_tiles``: the sum over the step's requests of ceil(rows / 16), which the caller knows from the rows per request
+extern "C" int fl_attn_mixed_tiled(const void* q, void* out, const void* cache_base, const int* positions, const int* block_table,
+                                   int max_blocks, const int* seq_q_start, const int* seq_q_len, int n_seqs, int n_tiles, int n,
+                                   int nh, int nkv, int hd, int page_size, int n_pages, float scale, int window, const float* slopes,
+                                   const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
+                                   hipStream_t stream) {
+    FL_CHECK(n >= 0 && nkv > 0 && nh % nkv == 0, "attn_mixed_tiled: bad head counts %d/%d", nh, nkv);
+    FL_CHECK(fl_attn_mixed_tiled_fits(nh, hd, page_size), "attn_mixed_tiled: %d heads of %d values over pages of %d are not what the kernel takes",
+             nh, hd, page_size);
+    FL_CHECK(window >= 0 && n_seqs >= 0 && n_tiles >= 0 && n_tiles <= n, "attn_mixed_tiled: bad window or tile count");
+    FL_CHECK(part_keys >= 0 && part_keys % AT_CHUNK == 0, "attn_mixed_tiled: parts of %d keys (a multiple of %d wanted)", part_keys, AT_CHUNK);
+    FL_CHECK(part_keys == 0 || (n_parts > 0 && n_parts <= 65535 && part_acc && part_ml), "attn_mixed_tiled: parts without their buffers");
+    if (n == 0 || n_tiles == 0) return 0;
+    PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
+    AttnMixed a{positions, nullptr, block_table, max_blocks, nh, scale, window, slopes, talk, sink,
+                part_keys, part_keys ? n_parts : 1, part_acc, part_ml};
+    AttnTiles tl{seq_q_start, seq_q_len, n_seqs};
+    const int HP = (nh + 15) & ~15;
+    const size_t lds = 4 * ((size_t)HP * AT_RAW_LD + (size_t)HP * AT_SC_LD + (size_t)HP * AT_ROWS);
+    dim3 grid(n_tiles, a.n_parts);
+#define FL_AT(DT)                                                                                                        \
+    do {                                                                                                                 \
+        static bool configured = false;                                                                                  \
+        if (!configured) {                                                                                               \
+            const hipError_t e = hipFuncSetAttribute((const void*)attn_mixed_tiled_kernel<DT>,                           \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);            \
+            FL_CHECK(e == hipSuccess, "attn_mixed_tiled: hipFuncSetAttribute failed: %s", hipGetErrorString(e));         \
+            configured = true;                                                                                           \
+        }                                                                                                                \
+        attn_mixed_tiled_kernel<DT><<<grid, AT_THREADS, lds, stream>>>((const bf16_t*)q, (bf16_t*)out, c, a, tl);        \
+    } while (0)
+    if (hd <= 32) FL_AT(2);
+    else if (hd <= 64) FL_AT(4);
+    else FL_AT(8);
+#undef FL_AT
+    FL_LAUNCH_CHECK();
+    if (part_keys > 0) {
+        attn_mixed_join_kernel<bf16_t><<<dim3(n, nh), 128, 0, stream>>>((bf16_t*)out, a, hd);
+        FL_LAUNCH_CHECK();
+    }
+    return 0;
+}
+FL_RECORDABLE(fl_attn_mixed_tiled)

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "fl_linear_scan_channel": [P, I, P, I, P, I, P, L, P, P, P, P, I, I, I, I, P],
     "fl_forget_gates": [P, I, I, I, P, P, P, P, I, I, P],
     "fl_attn_mixed": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, P, I, I, P, P, P],
+    "fl_attn_mixed_tiled": [P, P, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, P, P, P, I, I, P, P, P],
 }
 
 

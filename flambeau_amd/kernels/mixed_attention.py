@@ -1,7 +1,8 @@
 """The kernel set of attention whose heads' scores are mixed before the softmax (distance bias, mixing
-matrix, sink): every block of the kernel takes all heads of a query token.  The plain form gives a token
-to one block; the tuned form deals the keys of a step of few rows out to several blocks per token, as
-the split-K decode kernel of plain attention does, and joins the parts afterwards."""
+matrix, sink): every block of the kernels takes all heads of its query tokens.  The plain form gives a token
+to one block.  The tuned form runs bfloat16 caches on the matrix cores, 16 rows of a request per block, and deals
+the keys of a step of few rows out to several blocks per tile, as the split-K decode kernel of plain attention
+does, joining the parts afterwards; sizes the matrix-core kernel does not take go the plain way, with parts."""
 from __future__ import annotations
 
 import torch
@@ -9,8 +10,9 @@ import torch
 from . import ops
 from .sets import register_kernel_set
 
-PART_KEYS = 128       # keys per part (a multiple of the kernel's chunk), aligned to absolute positions
+PART_KEYS = 64        # keys per part (a multiple of the kernels' chunk), aligned to absolute positions
 FEW_ROWS = 64         # steps of up to this many rows deal their keys out
+TILE_ROWS = 16        # rows of a request that a block of the matrix-core kernel takes
 
 
 class PlainMixedAttention:
@@ -29,7 +31,7 @@ class TunedMixedAttention(PlainMixedAttention):
     def signature(self, batch, window: int):
         """The number of parts a token's keys are dealt out to (0: one block per token)."""
         ctx = batch.ctx_bound or batch.max_ctx_len
-        keys = min(window, ctx) if window else ctx
+        keys = min(window + TILE_ROWS - 1, ctx) if window else ctx          # (what the rows of a tile see together)
         if batch.n_tokens > FEW_ROWS or keys <= 2 * PART_KEYS:
             return 0
         parts = (keys - 1) // PART_KEYS + 2          # (a run of keys may begin anywhere inside its first part)
@@ -37,13 +39,17 @@ class TunedMixedAttention(PlainMixedAttention):
 
     def attention(self, q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink):
         parts = self.signature(step.host, window)
-        if not parts:
-            return super().attention(q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink)
         n, rt = q.shape[0], self.rt
-        acc = rt.buffer("amix_part_acc", n, parts * n_heads * kv.head_dim, torch.float32)
-        ml = rt.buffer("amix_part_ml", n, parts * n_heads * 2, torch.float32)
-        return ops.attn_mixed(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, slopes, talk, sink,
-                              part_keys=PART_KEYS, n_parts=parts, part_acc=acc, part_ml=ml)
+        split = {}
+        if parts:
+            split = dict(part_keys=PART_KEYS, n_parts=parts,
+                         part_acc=rt.buffer("amix_part_acc", n, parts * n_heads * kv.head_dim, torch.float32),
+                         part_ml=rt.buffer("amix_part_ml", n, parts * n_heads * 2, torch.float32))
+        if kv.pool.dtype == torch.bfloat16 and ops.attn_mixed_tiled_fits(n_heads, kv.head_dim, kv.page_size):
+            n_tiles = sum(-(-rows // TILE_ROWS) for rows in step.host.q_lens)
+            return ops.attn_mixed_tiled(q, out, kv, step.positions, table, step.seq_q_start, step.seq_q_len, n_tiles, n_heads, scale,
+                                        window, slopes, talk, sink, **split)
+        return ops.attn_mixed(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, slopes, talk, sink, **split)
 
 
 register_kernel_set("mixed_heads_attention", PlainMixedAttention, TunedMixedAttention)

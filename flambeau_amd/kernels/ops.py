@@ -771,3 +771,33 @@ def attn_mixed(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, 
          f(slopes, "slopes", (n_heads,)), f(talk, "talk", (n_heads, n_heads)), f(sink, "sink", (n_heads,)),
          int(part_keys), int(n_parts), f(part_acc, "part_acc", None), f(part_ml, "part_ml", None), stream_handle())
     return out
+
+
+def attn_mixed_tiled_fits(n_heads: int, head_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core form of the mixed-heads attention takes these sizes (bfloat16 caches only)."""
+    from .library import load
+    return bool(load().fl_attn_mixed_tiled_fits(int(n_heads), int(head_dim), int(page_size)))
+
+
+def attn_mixed_tiled(q, out, cache: PagedLayerCache, positions, block_table, seq_q_start, seq_q_len, n_tiles, n_heads, scale, window,
+                     slopes=None, talk=None, sink=None, part_keys: int = 0, n_parts: int = 1, part_acc=None, part_ml=None):
+    """``attn_mixed`` on the matrix cores: blocks take tiles of 16 rows of one request; ``n_tiles`` is the sum over
+    the requests of ceil(rows / 16), ``seq_q_start`` / ``seq_q_len`` the first row and the rows of every request."""
+    n = q.shape[0]
+    hd = cache.head_dim
+    dt = cache.pool.dtype
+    if dt != torch.bfloat16:
+        raise KernelError("attn_mixed_tiled: bfloat16 caches only")
+    S = seq_q_start.shape[0]
+    f = lambda t, name, shape: _check(t, "attn_mixed_tiled." + name, torch.float32, shape) if t is not None else None
+    if part_keys:
+        if part_acc is None or part_ml is None or part_acc.numel() < n * n_parts * n_heads * hd or part_ml.numel() < n * n_parts * n_heads * 2:
+            raise KernelError("attn_mixed_tiled: the parts' scratch is missing or too small")
+    call("fl_attn_mixed_tiled", _check(q, "attn_mixed_tiled.q", dt, (n, n_heads * hd)), _check(out, "attn_mixed_tiled.out", dt, (n, n_heads * hd)),
+         _check(cache.pool, "attn_mixed_tiled.cache"), _check(positions, "attn_mixed_tiled.positions", torch.int32, (n,)),
+         _check(block_table, "attn_mixed_tiled.block_table", torch.int32, (None, None)), block_table.shape[1],
+         _check(seq_q_start, "attn_mixed_tiled.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "attn_mixed_tiled.seq_q_len", torch.int32, (S,)),
+         S, int(n_tiles), n, int(n_heads), cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window),
+         f(slopes, "slopes", (n_heads,)), f(talk, "talk", (n_heads, n_heads)), f(sink, "sink", (n_heads,)),
+         int(part_keys), int(n_parts), f(part_acc, "part_acc", None), f(part_ml, "part_ml", None), stream_handle())
+    return out
