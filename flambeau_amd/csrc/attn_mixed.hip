@@ -292,11 +292,12 @@ FL_RECORDABLE(fl_attn_mixed)
 //   1. raw[g][query][key] = scale * Q_g . K^T - slope_g * (i - j)      v_mfma_f32_16x16x32_bf16, float into LDS;
 //      the (head, half chunk) tiles are dealt out to the waves, operands come straight from q and the pages
 //   2. score[h][pair] = sum_g talk[h][g] * raw[g][pair]                v_mfma_f32_16x16x4_f32 (true 32-bit): the
-//      mixing matrix is the A operand and lives in registers, 16 (query, key) pairs are a B operand's columns
+//      mixing matrix is the A operand, 16 (query, key) pairs are a B operand's columns, both read from LDS
 //   3. a thread per (head, query) row: mask, running maximum and sum (they stay in that thread's registers from
 //      chunk to chunk), weights as bfloat16 into LDS, and the factor by which the row's output shrinks
-//   4. out[h][query][:] = factor * out + P_h . V                        v_mfma_f32_16x16x32_bf16; a wave owns heads
-//      wave, wave + 8, ...; values lie transposed in a page, so eight keys of one dim are one 16-byte load
+//   4. out[h][query][:] = factor * out + P_h . V                        v_mfma_f32_16x16x32_bf16; a wave owns up to four
+//      consecutive heads in phases 1 and 4, and heads that share a key/value head share the operands read from the
+//      pages; values lie transposed in a page, so eight keys of one dim are one 16-byte load
 // Which block takes which tile is found from the step's own lists (first row and rows of every request).
 // With part_keys > 0 a tile's keys are dealt out to n_parts blocks as above and joined by the same kernel.
 #define AT_ROWS 16
@@ -322,6 +323,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     float* raw = lds;                                   // [HP][AT_RAW_LD]
     float* sc = raw + HP * AT_RAW_LD;                   // [HP][16][33]
     float* corr = sc + HP * AT_SC_LD;                   // [HP][16]
+    float* tk = corr + HP * AT_ROWS;                    // [HP][HP + 1]
     bf16_t* pb = (bf16_t*)raw;                          // [nh][16][AT_P_LD]: the weights take raw's place once it is mixed
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -366,15 +368,11 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     const bf16_t* kv = (const bf16_t*)cache.base;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    // ---- the mixing matrix as A operands: tA[hb][kk] = talk[16 hb + li][4 kk + lg] (the unit matrix without one)
-    float tA[2][AT_MAX_HEADS / 4];
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb)
-#pragma unroll
-        for (int kk = 0; kk < AT_MAX_HEADS / 4; ++kk) {
-            const int h = 16 * hb + li, g = 4 * kk + lg;
-            tA[hb][kk] = (h < nh && g < nh) ? (a.talk ? a.talk[h * nh + g] : (h == g ? 1.f : 0.f)) : 0.f;
-        }
+    // ---- the mixing matrix (the unit matrix without one), zeros around it up to a multiple of 16: A operands are read from here
+    for (int e = tid; e < HP * HP; e += AT_THREADS) {
+        const int h = e / HP, g = e % HP;
+        tk[h * (HP + 1) + g] = (h < nh && g < nh) ? (a.talk ? a.talk[h * nh + g] : (h == g ? 1.f : 0.f)) : 0.f;
+    }
     for (int e = tid; e < (HP - nh) * AT_RAW_LD; e += AT_THREADS) raw[nh * AT_RAW_LD + e] = 0.f;     // heads that do not exist
     // ---- the row (head, query) this thread keeps the softmax of
     const int rh = tid >> 4, rq = tid & 15;
@@ -387,31 +385,63 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     for (int hi = 0; hi < 4; ++hi)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[hi][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const int ksteps = (hd + 31) / 32;
+    constexpr int KS = (DT + 1) / 2;                     // steps of 32 dims in a score product
+    const int HPW = (nh + AT_WAVES - 1) / AT_WAVES;      // heads per wave, consecutive ones: at most 4
     __syncthreads();
 
     for (int base = (k0 / AT_CHUNK) * AT_CHUNK; base <= k1; base += AT_CHUNK) {
-        // ---- 1. raw scores of every head
-        for (int item = wave; item < 2 * nh; item += AT_WAVES) {
-            const int g = item >> 1, kt = item & 1;
-            const int jpos = base + 16 * kt + li;
-            int page = jpos <= p_last ? table[jpos / ps] : safe_page;
-            if (page < 0 || page >= cache.n_pages) page = safe_page;
-            const bf16_t* krow = kv + cache_k_offset(cache, page, g / group, jpos % ps, 0);
-            const bf16_t* qrow = q + ((size_t)(row0 + li) * nh + g) * hd;
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            for (int s = 0; s < ksteps; ++s) {
-                const int d = 32 * s + 8 * lg;
-                const bool in = d < hd;
-                const bf16x8 kf = in ? *(const bf16x8*)(krow + d) : zero8;
-                const bf16x8 qf = (in && li < cnt) ? *(const bf16x8*)(qrow + d) : zero8;
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf, kf, acc, 0, 0, 0);
-            }
-            const float slope = a.slopes ? a.slopes[g] : 0.f;
+        // ---- 1. raw scores: a wave takes HPW consecutive heads
+        {
+            const size_t head_stride = (size_t)ps * hd;
+            const bf16_t* kpage[2];
+            int jpos[2];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int qq = 4 * lg + r;
-                raw[g * AT_RAW_LD + qq * AT_CHUNK + 16 * kt + li] = acc[r] * a.scale - slope * (float)(p_first + qq - jpos);
+            for (int kt = 0; kt < 2; ++kt) {
+                jpos[kt] = base + 16 * kt + li;
+                int page = jpos[kt] <= p_last ? table[jpos[kt] / ps] : safe_page;
+                if (page < 0 || page >= cache.n_pages) page = safe_page;
+                kpage[kt] = kv + cache_k_offset(cache, page, 0, jpos[kt] % ps, 0);
+            }
+            // the keys of a key/value head are loaded once for the heads that share it (they follow one another in a
+            // wave)
+            auto load_q = [&](int g, bf16x8* qf) {
+                const bf16_t* qrow = q + ((size_t)(row0 + li) * nh + g) * hd;
+#pragma unroll
+                for (int s = 0; s < KS; ++s) {
+                    const int d = 32 * s + 8 * lg;
+                    qf[s] = (d < hd && li < cnt && g < nh) ? *(const bf16x8*)(qrow + d) : zero8;
+                }
+            };
+            bf16x8 kf[2][KS], qf[KS];
+            int kvh_held = -1;
+#pragma unroll
+            for (int hi = 0; hi < 4; ++hi) {
+                const int g = wave * HPW + hi;
+                if (hi >= HPW || g >= nh) continue;
+                const int kvh = g / group;
+                if (kvh != kvh_held) {
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                        for (int s = 0; s < KS; ++s) {
+                            const int d = 32 * s + 8 * lg;
+                            kf[kt][s] = d < hd ? *(const bf16x8*)(kpage[kt] + kvh * head_stride + d) : zero8;
+                        }
+                    kvh_held = kvh;
+                }
+                load_q(g, qf);
+                const float slope = a.slopes ? a.slopes[g] : 0.f;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[s], kf[kt][s], acc, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int qq = 4 * lg + r;
+                        raw[g * AT_RAW_LD + qq * AT_CHUNK + 16 * kt + li] = acc[r] * a.scale - slope * (float)(p_first + qq - jpos[kt]);
+                    }
+                }
             }
         }
         __syncthreads();
@@ -424,7 +454,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
 #pragma unroll
                 for (int kk = 0; kk < AT_MAX_HEADS / 4; ++kk) {
                     if (4 * kk >= HP) continue;
-                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(tA[hb][kk], raw[(4 * kk + lg) * AT_RAW_LD + 16 * pt + li], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(tk[(16 * hb + li) * (HP + 1) + 4 * kk + lg], raw[(4 * kk + lg) * AT_RAW_LD + 16 * pt + li], c, 0, 0, 0);
                 }
                 const int pair = 16 * pt + li;
 #pragma unroll
@@ -446,11 +476,11 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
                 corr[rh * AT_ROWS + rq] = 1.f;
             } else {
                 const float m_new = fmaxf(rm, mx);
-                const float cr = rm == -INFINITY ? 0.f : expf(rm - m_new);
+                const float cr = rm == -INFINITY ? 0.f : __expf(rm - m_new);
                 float sum = 0.f;
                 for (int j = 0; j < AT_CHUNK; j += 2) {
-                    const float e0 = (base + j >= r_lo && base + j <= r_hi) ? expf(srow[j] - m_new) : 0.f;
-                    const float e1 = (base + j + 1 >= r_lo && base + j + 1 <= r_hi) ? expf(srow[j + 1] - m_new) : 0.f;
+                    const float e0 = (base + j >= r_lo && base + j <= r_hi) ? __expf(srow[j] - m_new) : 0.f;
+                    const float e1 = (base + j + 1 >= r_lo && base + j + 1 <= r_hi) ? __expf(srow[j + 1] - m_new) : 0.f;
                     sum += e0 + e1;
                     const bf16_t b0 = (bf16_t)e0, b1 = (bf16_t)e1;
                     prow[j >> 1] = (unsigned)__builtin_bit_cast(unsigned short, b0) | ((unsigned)__builtin_bit_cast(unsigned short, b1) << 16);
@@ -462,31 +492,50 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
         }
         __syncthreads();
         // ---- 4. the weighted sums of the values
-#pragma unroll
-        for (int hi = 0; hi < 4; ++hi) {
-            const int h = wave + AT_WAVES * hi;
-            if (h >= nh) continue;
-            float cr[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) cr[r] = corr[h * AT_ROWS + 4 * lg + r];
-            const bf16x8 pf = *(const bf16x8*)(pb + (h * AT_ROWS + li) * AT_P_LD + 8 * lg);
+        {
             const int jr = base + 8 * lg;                                      // this lane's run of eight keys
             int page = jr <= p_last ? table[jr / ps] : -1;
             const bool run_on = page >= 0 && page < cache.n_pages && jr <= k1;
             if (!run_on) page = safe_page;
-            const bf16_t* vbase = kv + cache_v_offset(cache, page, h / group, jr % ps, 0);
+            const bf16_t* vpage = kv + cache_v_offset(cache, page, 0, jr % ps, 0);
+            const size_t head_stride = (size_t)ps * hd;
+            constexpr int DH = DT / 2;                                         // the value dims in two halves: fewer operands held at a time
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const int d = 16 * dt + li;
-                bf16x8 vf = (run_on && d < hd) ? *(const bf16x8*)(vbase + (size_t)d * ps) : zero8;
-                if (jr + 7 > k1) {                                             // keys that nobody wrote yet may hold anything
+            for (int half = 0; half < 2; ++half) {
+                bf16x8 vf[DH];
+                int kvh_held = -1;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (jr + e > k1) vf[e] = (bf16_t)0.f;
+                for (int hi = 0; hi < 4; ++hi) {
+                    const int h = wave * HPW + hi;
+                    if (hi >= HPW || h >= nh) continue;
+                    const int kvh = h / group;
+                    if (kvh != kvh_held) {
+                        const bf16_t* vbase = vpage + kvh * head_stride;
+#pragma unroll
+                        for (int dt = 0; dt < DH; ++dt) {
+                            const int d = 16 * (half * DH + dt) + li;
+                            vf[dt] = (run_on && d < hd) ? *(const bf16x8*)(vbase + (size_t)d * ps) : zero8;
+                        }
+                        if (jr + 7 > k1) {                                     // keys that nobody wrote yet may hold anything
+#pragma unroll
+                            for (int dt = 0; dt < DH; ++dt)
+#pragma unroll
+                                for (int e = 0; e < 8; ++e)
+                                    if (jr + e > k1) vf[dt][e] = (bf16_t)0.f;
+                        }
+                        kvh_held = kvh;
+                    }
+                    float cr[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) cr[r] = corr[h * AT_ROWS + 4 * lg + r];
+                    const bf16x8 pf = *(const bf16x8*)(pb + (h * AT_ROWS + li) * AT_P_LD + 8 * lg);
+#pragma unroll
+                    for (int dt = 0; dt < DH; ++dt) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[hi][half * DH + dt][r] *= cr[r];
+                        o[hi][half * DH + dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[hi][half * DH + dt], 0, 0, 0);
+                    }
                 }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) o[hi][dt][r] *= cr[r];
-                o[hi][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[hi][dt], 0, 0, 0);
             }
         }
         __syncthreads();
@@ -506,8 +555,8 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     __syncthreads();
 #pragma unroll
     for (int hi = 0; hi < 4; ++hi) {
-        const int h = wave + AT_WAVES * hi;
-        if (h >= nh) continue;
+        const int h = wave * HPW + hi;
+        if (hi >= HPW || h >= nh) continue;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int qq = 4 * lg + r;
@@ -554,7 +603,7 @@ extern "C" int fl_attn_mixed_tiled(const void* q, void* out, const void* cache_b
                 part_keys, part_keys ? n_parts : 1, part_acc, part_ml};
     AttnTiles tl{seq_q_start, seq_q_len, n_seqs};
     const int HP = (nh + 15) & ~15;
-    const size_t lds = 4 * ((size_t)HP * AT_RAW_LD + (size_t)HP * AT_SC_LD + (size_t)HP * AT_ROWS);
+    const size_t lds = 4 * ((size_t)HP * AT_RAW_LD + (size_t)HP * AT_SC_LD + (size_t)HP * AT_ROWS + (size_t)HP * (HP + 1));
     dim3 grid(n_tiles, a.n_parts);
 #define FL_AT(DT)                                                                                                        \
     do {                                                                                                                 \

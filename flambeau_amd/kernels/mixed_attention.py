@@ -10,9 +10,11 @@ import torch
 from . import ops
 from .sets import register_kernel_set
 
-PART_KEYS = 64        # keys per part (a multiple of the kernels' chunk), aligned to absolute positions
-FEW_ROWS = 64         # steps of up to this many rows deal their keys out
+PART_KEYS = 64        # keys per part of a step of few rows (a multiple of the kernels' chunk), aligned to absolute positions
+FEW_ROWS = 64         # steps of up to this many rows deal their keys out that finely
 TILE_ROWS = 16        # rows of a request that a block of the matrix-core kernel takes
+PROMPT_PART_KEYS = 512    # keys per part of a larger step whose tiles alone do not fill the chip
+FULL_CHIP_TILES = 512     # from this many tiles on nothing is dealt out
 
 
 class PlainMixedAttention:
@@ -29,20 +31,26 @@ class PlainMixedAttention:
 
 class TunedMixedAttention(PlainMixedAttention):
     def signature(self, batch, window: int):
-        """The number of parts a token's keys are dealt out to (0: one block per token)."""
+        """``(keys per part, parts)`` a tile's keys are dealt out to; ``(0, 0)``: one block finishes a tile."""
         ctx = batch.ctx_bound or batch.max_ctx_len
         keys = min(window + TILE_ROWS - 1, ctx) if window else ctx          # (what the rows of a tile see together)
-        if batch.n_tokens > FEW_ROWS or keys <= 2 * PART_KEYS:
-            return 0
-        parts = (keys - 1) // PART_KEYS + 2          # (a run of keys may begin anywhere inside its first part)
-        return 1 << (parts - 1).bit_length()
+        if batch.n_tokens <= FEW_ROWS:
+            part_keys = PART_KEYS
+        elif sum(-(-rows // TILE_ROWS) for rows in batch.q_lens) < FULL_CHIP_TILES:
+            part_keys = PROMPT_PART_KEYS
+        else:
+            return (0, 0)
+        if keys <= 2 * part_keys:
+            return (0, 0)
+        parts = (keys - 1) // part_keys + 2          # (a run of keys may begin anywhere inside its first part)
+        return (part_keys, 1 << (parts - 1).bit_length())
 
     def attention(self, q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink):
-        parts = self.signature(step.host, window)
+        part_keys, parts = self.signature(step.host, window)
         n, rt = q.shape[0], self.rt
         split = {}
         if parts:
-            split = dict(part_keys=PART_KEYS, n_parts=parts,
+            split = dict(part_keys=part_keys, n_parts=parts,
                          part_acc=rt.buffer("amix_part_acc", n, parts * n_heads * kv.head_dim, torch.float32),
                          part_ml=rt.buffer("amix_part_ml", n, parts * n_heads * 2, torch.float32))
         if kv.pool.dtype == torch.bfloat16 and ops.attn_mixed_tiled_fits(n_heads, kv.head_dim, kv.page_size):

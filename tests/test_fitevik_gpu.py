@@ -360,7 +360,7 @@ def test_single_tokens_behind_a_long_window_deal_their_keys_out():
         mixer.kernels.signature = lambda batch, w, k=mixer.kernels: seen.append(orig(k, batch, w)) or seen[-1]
         got = run_mixer(mixer, rt, x, [n - 20, 3] + [1] * 17, page_size=16, n_pages=64)
         del mixer.kernels.signature
-        assert max(seen) >= 4 and seen[0] == 0               # the prompt: a block per token; the single tokens: parts
+        assert seen[0] == (0, 0) and max(seen)[1] >= 4       # the prompt: one block per tile; the single tokens: parts of 64 keys
         assert np.abs(got[n - 20:] - want).max() < 3e-2 * np.abs(want).max(), window
 
 
