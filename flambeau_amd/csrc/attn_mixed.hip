@@ -317,7 +317,7 @@ template <int DT>
 __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                                                                        PagedCache cache, AttnMixed a, AttnTiles tl) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    __shared__ int s_tile[3];
+    __shared__ int s_tile[4];
     const int nh = a.nh, hd = cache.head_dim, ps = cache.page_size;
     const int HP = (nh + 15) & ~15;
     float* raw = lds;                                   // [HP][AT_RAW_LD]
@@ -329,17 +329,31 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
 
-    // ---- which rows: tile blockIdx.x of the requests' portions, 16 rows each
-    if (tid == 0) {
-        int t = blockIdx.x, seq = -1, row0 = 0, cnt = 0;
-        for (int s = 0; s < tl.n_seqs; ++s) {
-            const int len = tl.seq_q_len[s], nt = (len + AT_ROWS - 1) / AT_ROWS;
-            if (t < nt) { seq = s; row0 = tl.seq_q_start[s] + AT_ROWS * t; cnt = min(AT_ROWS, len - AT_ROWS * t); break; }
-            t -= nt;
+    // ---- which rows: tile blockIdx.x of the requests' portions, 16 rows each (the requests' row counts are fetched by
+    // all threads at once, then one thread walks them in LDS)
+    int* s_len = (int*)lds;
+    for (int s0 = 0, t = blockIdx.x, done = 0; s0 < tl.n_seqs && !done; s0 += AT_THREADS) {
+        const int ns = min(AT_THREADS, tl.n_seqs - s0);
+        if (tid < ns) s_len[tid] = tl.seq_q_len[s0 + tid];
+        if (tid == 0) s_tile[0] = -1;
+        __syncthreads();
+        if (tid == 0) {
+            for (int s = 0; s < ns; ++s) {
+                const int len = s_len[s], nt = (len + AT_ROWS - 1) / AT_ROWS;
+                if (t < nt) {
+                    s_tile[0] = s0 + s; s_tile[1] = tl.seq_q_start[s0 + s] + AT_ROWS * t; s_tile[2] = min(AT_ROWS, len - AT_ROWS * t);
+                    break;
+                }
+                t -= nt;
+            }
+            s_tile[3] = t;
         }
-        s_tile[0] = seq; s_tile[1] = row0; s_tile[2] = cnt;
+        __syncthreads();
+        done = s_tile[0] >= 0;
+        t = s_tile[3];
+        __syncthreads();
     }
-    __syncthreads();
+    if (tl.n_seqs <= 0) return;
     const int seq = s_tile[0], row0 = s_tile[1], cnt = s_tile[2];
     if (seq < 0) return;
     const int p_first = a.positions[row0], p_last = p_first + cnt - 1;

@@ -94,6 +94,24 @@ def test_layer_norm_ahead_and_behind(dtype, W):
     assert torch.allclose(o, norm.bias.expand(2, W), atol=1e-6)
 
 
+@pytest.mark.parametrize("W", [256, 4096, 1000])
+def test_layer_norm_bits_do_not_depend_on_the_step_s_size(W):
+    """A step of few rows keeps its rows in registers, a large one reads them three times: the same sums in the
+    same order, so a row's bits are the same in both."""
+    from flambeau_amd.kernels import ops
+    g = torch.Generator().manual_seed(W)
+    x = (torch.randn(300, W, generator=g) * 2 + 0.5).to(DEV)
+    d = torch.randn(300, W, generator=g).to(DEV)
+    w, b = (1 + 0.1 * torch.randn(W, generator=g)).to(DEV), torch.randn(W, generator=g).to(DEV)
+    big = ops.layernorm(x, w, b, torch.empty(300, W, device=DEV), 1e-5, delta=d)
+    few = ops.layernorm(x[:7].contiguous(), w, b, torch.empty(7, W, device=DEV), 1e-5, delta=d[:7].contiguous())
+    assert torch.equal(big[:7], few)
+    r_big, r_few = x.clone(), x[:7].clone()
+    ops.layernorm_add(d, w, b, r_big, 1e-5)
+    ops.layernorm_add(d[:7].contiguous(), w, b, r_few, 1e-5)
+    assert torch.equal(r_big[:7], r_few)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_embedding_with_learned_positions_and_the_scaled_head(dtype):
     from flambeau_amd.parts import EMBEDDINGS, HEADS, PartSpec
