@@ -394,6 +394,8 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     const int rp = p_first + rq;
     const int r_lo = max(k0, a.window > 0 ? rp - a.window + 1 : 0), r_hi = min(k1, rp);
     float rm = -INFINITY, rl = 0.f;
+    // keys that every row of the tile sees: from the last row's first key to the first row's position, inside this block's part
+    const int all_lo = max(k0, a.window > 0 ? p_last - a.window + 1 : 0), all_hi = min(k1, p_first);
     f32x4 o[4][DT];
 #pragma unroll
     for (int hi = 0; hi < 4; ++hi)
@@ -477,31 +479,56 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
             }
         }
         __syncthreads();
-        // ---- 3. the rows' softmax
+        // ---- 3. the rows' softmax.  Most chunks lie inside every row's window: there no key is tested
         if (rh < nh) {
             unsigned* prow = (unsigned*)(pb + (rh * AT_ROWS + rq) * AT_P_LD);
             const float* srow = sc + rh * AT_SC_LD + rq * (AT_CHUNK + 1);
-            float mx = -INFINITY;
-            if (row_on)
-                for (int j = 0; j < AT_CHUNK; ++j)
-                    if (base + j >= r_lo && base + j <= r_hi) mx = fmaxf(mx, srow[j]);
-            if (mx == -INFINITY) {                                            // no key of this chunk for this row
-                for (int j2 = 0; j2 < AT_CHUNK / 2; ++j2) prow[j2] = 0u;
-                corr[rh * AT_ROWS + rq] = 1.f;
-            } else {
+            const bool inside = base >= all_lo && base + AT_CHUNK - 1 <= all_hi;     // (the same for the whole block)
+            auto pack = [](float e0, float e1) {
+                const bf16_t b0 = (bf16_t)e0, b1 = (bf16_t)e1;
+                return (unsigned)__builtin_bit_cast(unsigned short, b0) | ((unsigned)__builtin_bit_cast(unsigned short, b1) << 16);
+            };
+            if (inside && row_on) {
+                float sv[AT_CHUNK];
+#pragma unroll
+                for (int j = 0; j < AT_CHUNK; ++j) sv[j] = srow[j];
+                float mx = sv[0];
+#pragma unroll
+                for (int j = 1; j < AT_CHUNK; ++j) mx = fmaxf(mx, sv[j]);
                 const float m_new = fmaxf(rm, mx);
                 const float cr = rm == -INFINITY ? 0.f : __expf(rm - m_new);
                 float sum = 0.f;
+#pragma unroll
                 for (int j = 0; j < AT_CHUNK; j += 2) {
-                    const float e0 = (base + j >= r_lo && base + j <= r_hi) ? __expf(srow[j] - m_new) : 0.f;
-                    const float e1 = (base + j + 1 >= r_lo && base + j + 1 <= r_hi) ? __expf(srow[j + 1] - m_new) : 0.f;
+                    const float e0 = __expf(sv[j] - m_new), e1 = __expf(sv[j + 1] - m_new);
                     sum += e0 + e1;
-                    const bf16_t b0 = (bf16_t)e0, b1 = (bf16_t)e1;
-                    prow[j >> 1] = (unsigned)__builtin_bit_cast(unsigned short, b0) | ((unsigned)__builtin_bit_cast(unsigned short, b1) << 16);
+                    prow[j >> 1] = pack(e0, e1);
                 }
                 rl = rl * cr + sum;
                 rm = m_new;
                 corr[rh * AT_ROWS + rq] = cr;
+            } else {
+                float mx = -INFINITY;
+                if (row_on)
+                    for (int j = 0; j < AT_CHUNK; ++j)
+                        if (base + j >= r_lo && base + j <= r_hi) mx = fmaxf(mx, srow[j]);
+                if (mx == -INFINITY) {                                        // no key of this chunk for this row
+                    for (int j2 = 0; j2 < AT_CHUNK / 2; ++j2) prow[j2] = 0u;
+                    corr[rh * AT_ROWS + rq] = 1.f;
+                } else {
+                    const float m_new = fmaxf(rm, mx);
+                    const float cr = rm == -INFINITY ? 0.f : __expf(rm - m_new);
+                    float sum = 0.f;
+                    for (int j = 0; j < AT_CHUNK; j += 2) {
+                        const float e0 = (base + j >= r_lo && base + j <= r_hi) ? __expf(srow[j] - m_new) : 0.f;
+                        const float e1 = (base + j + 1 >= r_lo && base + j + 1 <= r_hi) ? __expf(srow[j + 1] - m_new) : 0.f;
+                        sum += e0 + e1;
+                        prow[j >> 1] = pack(e0, e1);
+                    }
+                    rl = rl * cr + sum;
+                    rm = m_new;
+                    corr[rh * AT_ROWS + rq] = cr;
+                }
             }
         }
         __syncthreads();
