@@ -304,8 +304,9 @@ FL_RECORDABLE(fl_attn_mixed)
 #define AT_CHUNK 32
 #define AT_THREADS 512
 #define AT_WAVES 8
-#define AT_RAW_LD (AT_ROWS * AT_CHUNK + 16)     // floats per head of raw (the 16 spread the four heads of an operand over the banks)
-#define AT_SC_LD (AT_ROWS * (AT_CHUNK + 1))     // floats per head of score: rows of 33
+#define AT_RAW_Q (AT_CHUNK + 4)                 // floats per query row of raw: the four row groups of a score tile fall on two bank halves
+#define AT_RAW_LD (AT_ROWS * AT_RAW_Q + 16)     // floats per head of raw (the 16 spread the four heads of an operand over the banks)
+#define AT_SC_LD (AT_ROWS * (AT_CHUNK + 1) + 4) // floats per head of score: rows of 33 (a thread walks a row), heads four apart on two bank halves
 #define AT_P_LD 40                              // bfloat16 per row of weights
 #define AT_MAX_HEADS 32
 
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int qq = 4 * lg + r;
-                        raw[g * AT_RAW_LD + qq * AT_CHUNK + 16 * kt + li] = acc[r] * a.scale - slope * (float)(p_first + qq - jpos[kt]);
+                        raw[g * AT_RAW_LD + qq * AT_RAW_Q + 16 * kt + li] = acc[r] * a.scale - slope * (float)(p_first + qq - jpos[kt]);
                     }
                 }
             }
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
 #pragma unroll
                 for (int kk = 0; kk < AT_MAX_HEADS / 4; ++kk) {
                     if (4 * kk >= HP) continue;
-                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(tk[(16 * hb + li) * (HP + 1) + 4 * kk + lg], raw[(4 * kk + lg) * AT_RAW_LD + 16 * pt + li], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(tk[(16 * hb + li) * (HP + 1) + 4 * kk + lg], raw[(4 * kk + lg) * AT_RAW_LD + (pt >> 1) * AT_RAW_Q + 16 * (pt & 1) + li], c, 0, 0, 0);
                 }
                 const int pair = 16 * pt + li;
 #pragma unroll
@@ -481,7 +482,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
         __syncthreads();
         // ---- 3. the rows' softmax.  Most chunks lie inside every row's window: there no key is tested
         if (rh < nh) {
-            unsigned* prow = (unsigned*)(pb + (rh * AT_ROWS + rq) * AT_P_LD);
+            u32x4* prow4 = (u32x4*)(pb + (rh * AT_ROWS + rq) * AT_P_LD);      // eight weights a store
             const float* srow = sc + rh * AT_SC_LD + rq * (AT_CHUNK + 1);
             const bool inside = base >= all_lo && base + AT_CHUNK - 1 <= all_hi;     // (the same for the whole block)
             auto pack = [](float e0, float e1) {
@@ -499,10 +500,15 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
                 const float cr = rm == -INFINITY ? 0.f : __expf(rm - m_new);
                 float sum = 0.f;
 #pragma unroll
-                for (int j = 0; j < AT_CHUNK; j += 2) {
-                    const float e0 = __expf(sv[j] - m_new), e1 = __expf(sv[j + 1] - m_new);
-                    sum += e0 + e1;
-                    prow[j >> 1] = pack(e0, e1);
+                for (int j8 = 0; j8 < AT_CHUNK; j8 += 8) {
+                    u32x4 w;
+#pragma unroll
+                    for (int j = 0; j < 8; j += 2) {
+                        const float e0 = __expf(sv[j8 + j] - m_new), e1 = __expf(sv[j8 + j + 1] - m_new);
+                        sum += e0 + e1;
+                        w[j >> 1] = pack(e0, e1);
+                    }
+                    prow4[j8 >> 3] = w;
                 }
                 rl = rl * cr + sum;
                 rm = m_new;
@@ -513,17 +519,23 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
                     for (int j = 0; j < AT_CHUNK; ++j)
                         if (base + j >= r_lo && base + j <= r_hi) mx = fmaxf(mx, srow[j]);
                 if (mx == -INFINITY) {                                        // no key of this chunk for this row
-                    for (int j2 = 0; j2 < AT_CHUNK / 2; ++j2) prow[j2] = 0u;
+                    for (int j8 = 0; j8 < AT_CHUNK / 8; ++j8) prow4[j8] = (u32x4){0u, 0u, 0u, 0u};
                     corr[rh * AT_ROWS + rq] = 1.f;
                 } else {
                     const float m_new = fmaxf(rm, mx);
                     const float cr = rm == -INFINITY ? 0.f : __expf(rm - m_new);
                     float sum = 0.f;
-                    for (int j = 0; j < AT_CHUNK; j += 2) {
-                        const float e0 = (base + j >= r_lo && base + j <= r_hi) ? __expf(srow[j] - m_new) : 0.f;
-                        const float e1 = (base + j + 1 >= r_lo && base + j + 1 <= r_hi) ? __expf(srow[j + 1] - m_new) : 0.f;
-                        sum += e0 + e1;
-                        prow[j >> 1] = pack(e0, e1);
+                    for (int j8 = 0; j8 < AT_CHUNK; j8 += 8) {
+                        u32x4 w;
+#pragma unroll
+                        for (int j = 0; j < 8; j += 2) {
+                            const int jp = base + j8 + j;
+                            const float e0 = (jp >= r_lo && jp <= r_hi) ? __expf(srow[j8 + j] - m_new) : 0.f;
+                            const float e1 = (jp + 1 >= r_lo && jp + 1 <= r_hi) ? __expf(srow[j8 + j + 1] - m_new) : 0.f;
+                            sum += e0 + e1;
+                            w[j >> 1] = pack(e0, e1);
+                        }
+                        prow4[j8 >> 3] = w;
                     }
                     rl = rl * cr + sum;
                     rm = m_new;
