@@ -225,7 +225,7 @@ __global__ __launch_bounds__(128) void attn_mixed_join_kernel(T* __restrict__ ou
         float den = a.sink ? expf(sk - top) : 0.f, num = 0.f;
         for (int part = 0; part < a.n_parts; ++part) {
             const float m = pm[(part * nh + h) * 2], l = pm[(part * nh + h) * 2 + 1];
-            if (!(l > 0.f)) continue;                                         // a part without keys
+            if (!(l > 0.f)) continue;                                         // a part without keys: what it holds is not read
             const float f = expf(m - top);
             den = fmaf(l, f, den);
             num = fmaf(a.part_acc[(((size_t)token * a.n_parts + part) * nh + h) * hd + d], f, num);

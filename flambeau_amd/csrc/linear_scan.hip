@@ -212,7 +212,8 @@ __global__ __launch_bounds__(256) void forget_gates_kernel(const float* __restri
                                                            const float* __restrict__ bias, const float* __restrict__ lower,
                                                            float* __restrict__ q_out, float* __restrict__ f_out, int HD) {
     const float* row = proj + (size_t)blockIdx.x * ld;
-    for (int i = threadIdx.x; i < HD; i += 256) {
+    const int i = blockIdx.y * 256 + threadIdx.x;          // (a value per thread: a step of few tokens still fills units)
+    if (i < HD) {
         const float zq = row[col_q + i];
         q_out[(size_t)blockIdx.x * HD + i] = zq / (1.0f + expf(-zq));
         const float low = lower ? lower[i] : 0.f;
@@ -225,7 +226,7 @@ extern "C" int fl_forget_gates(const float* proj, int ld, int col_q, int col_f, 
                                float* q_out, float* f_out, int n, int HD, hipStream_t stream) {
     FL_CHECK(n >= 0 && HD > 0 && ld >= col_q + HD && ld >= col_f + HD && col_q >= 0 && col_f >= 0, "forget_gates: columns beyond rows %d wide", ld);
     if (n == 0) return 0;
-    forget_gates_kernel<<<n, 256, 0, stream>>>(proj, ld, col_q, col_f, bias, lower, q_out, f_out, HD);
+    forget_gates_kernel<<<dim3(n, (HD + 255) / 256), 256, 0, stream>>>(proj, ld, col_q, col_f, bias, lower, q_out, f_out, HD);
     FL_LAUNCH_CHECK();
     return 0;
 }
