@@ -54,8 +54,9 @@ def _attention(m: KeyReader, index: int, before: list) -> WindowAttentionConfig:
     heads, kv_heads = m.integer("heads", minimum=1), m.integer("kv_heads", minimum=1)
     if heads % kv_heads:
         raise ConfigError(f"{m.where}: {heads} heads are not a multiple of {kv_heads} key/value heads")
+    mask = m.section("mask", default=None)                    # (a mixer without a mask sees every earlier token: window 0)
     cfg = WindowAttentionConfig(heads=heads, kv_heads=kv_heads, dim=m.integer("dim", minimum=1), vdim=m.integer("vdim", minimum=1),
-                                scale=m.number("scale", positive=True), window=m.section("mask").integer("size", minimum=1),
+                                scale=m.number("scale", positive=True), window=mask.integer("size", minimum=1) if mask is not None else 0,
                                 kv_from=m.integer("kv_from", default=None, minimum=0))
     if cfg.kv_from is not None:
         src = before[cfg.kv_from].mixer if cfg.kv_from < index else None

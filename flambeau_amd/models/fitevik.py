@@ -64,12 +64,13 @@ def _feed_forward(cfg: FitevikConfig, f, p: str):
 
 def fitevik_spec(cfg: FitevikConfig) -> ModelSpec:
     norm = PartSpec("layernorm", dict(hidden_size=cfg.width, eps=cfg.eps))
-    # a cache keeps what the widest window among the layers that read it needs
+    # a cache keeps what the widest window among the layers that read it needs (0: everything, where one of them has no window)
     cache_windows: dict = {}
     for l, layer in enumerate(cfg.layers):
         if isinstance(layer.mixer, WindowAttentionConfig):
             owner = l if layer.mixer.kv_from is None else layer.mixer.kv_from
-            cache_windows[owner] = max(cache_windows.get(owner, 0), layer.mixer.window)
+            kept, window = cache_windows.get(owner), layer.mixer.window
+            cache_windows[owner] = window if kept is None else (0 if kept == 0 or window == 0 else max(kept, window))
     layers, run_order = [], []
     for l, layer in enumerate(cfg.layers):
         p = f"l{l}."

@@ -5,7 +5,7 @@ one to eight query heads per key/value head, key and value sizes that differ eit
 of 8, windows of one key, of a few, across several pages and beyond 256 keys, layers that read the keys and
 values of an earlier layer through a narrower, an equal and a wider window, one, some and all experts per
 token, layers without a feed-forward, a logit scale that is no power of two or absent, widths and vocabularies
-that are no multiples of 8."""
+that are no multiples of 8, mixers without a mask."""
 import json
 
 import torch
@@ -18,7 +18,9 @@ def hgrn(heads, dim, vdim):
 
 
 def att(heads, kv_heads, dim, vdim, scale, window, kv_from=None):
-    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, mask={"size": window})
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if window is not None:                  # (None: no mask, every earlier key is seen)
+        m["mask"] = {"size": window}
     if kv_from is not None:
         m["kv_from"] = kv_from
     return {"type": "attention", "mixer": m}
@@ -72,6 +74,13 @@ CONFIGS = {
         (att(4, 2, 16, 16, 0.4, 50, kv_from=0), moe(4, 2, 24)),
         (att(3, 3, 8, 12, 0.5, 9), dense(24)),
     ]), seed=41, std=0.15, page_size=16),
+    # mixers without a mask: a reader that sees every key of a source whose own window is narrow, and a layer of its own
+    "P": dict(config=model(70, 32, 1e-5, 1.5, 300, [
+        (att(4, 2, 16, 16, 0.3, 11), dense(24)),
+        (hgrn(2, 8, 8), None),
+        (att(4, 2, 16, 16, 0.35, None, kv_from=0), moe(3, 2, 8)),
+        (att(2, 1, 8, 24, 0.4, None), dense(16)),
+    ]), seed=51, std=0.18, page_size=16),
 }
 
 STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}

@@ -109,13 +109,18 @@ def mixed_softmax_attention(q, k, v, window, scale, slopes, talk, sink, first=0)
     return out
 
 
+def window_of(m):
+    """Keys a query sees, its own included; 0 (every earlier key) where the mixer has no mask."""
+    return m["mask"]["size"] if m.get("mask") else 0
+
+
 def attention(h, m, t, p, eps, k, v):
     """Softmax attention inside a sliding window with a distance bias, scores mixed over the heads, and a
     sink in the denominator.  ``k`` [T, G, dim], ``v`` [T, G, vdim]: this layer's or another's."""
     T = h.shape[0]
     H, D = m["heads"], m["dim"]
     q = rms_norm(h @ t[p + "q"].T, t[p + "q.norm"], eps).reshape(T, H, D)
-    out = mixed_softmax_attention(q, k, v, m["mask"]["size"], m["scale"], head_slopes(H), t[p + "talk"], t[p + "sink"])
+    out = mixed_softmax_attention(q, k, v, window_of(m), m["scale"], head_slopes(H), t[p + "talk"], t[p + "sink"])
     return out.reshape(T, -1) @ t[p + "o"].T
 
 

@@ -111,6 +111,24 @@ def test_parts_caches_and_names():
     assert shares == [None, None, None, 2, 2] and specs[2] == PagedKVSpec(2, 32, 64) and specs[0] == PagedKVSpec(1, 16, 1)
 
 
+def test_a_mixer_without_a_mask_sees_everything():
+    """No ``mask``: window 0; a cache that such a layer reads keeps every key, whatever window its owner has."""
+    from flambeau_amd.models.decoder import DecoderModel
+    from flambeau_amd.parts import PagedKVSpec
+    from flambeau_amd.registry import config_from_dict
+    raw = json.loads(json.dumps(CONFIGS["K"]["config"]))
+    del raw["layers"][2]["mixer"]["mask"]                      # the reader of layer 1, whose own window is 13
+    del raw["layers"][4]["mixer"]["mask"]
+    arch, cfg = config_from_dict(raw, "test")
+    assert cfg.layers[2].mixer.window == 0 and cfg.layers[1].mixer.window == 13
+    model = DecoderModel(arch.build_spec(cfg), rt=None)
+    specs, _ = model.cache_entries()
+    assert specs[1] == PagedKVSpec(2, 16, 0) and specs[4] == PagedKVSpec(4, 24, 0)
+    assert [b.mixer.window for b in model.blocks if hasattr(b.mixer, "own_kv")] == [13, 0, 0]
+    # the plain side reads the same file the same way
+    assert pf.window_of(raw["layers"][2]["mixer"]) == 0 and pf.window_of(raw["layers"][1]["mixer"]) == 13
+
+
 def test_random_weights_as_a_folder(tmp_path):
     from flambeau_amd.models.decoder import DecoderModel
     from flambeau_amd.weights.loader import SafetensorsDir, check_against_manifest

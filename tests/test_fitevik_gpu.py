@@ -407,7 +407,7 @@ def test_the_stream_after_every_layer(dirs, name, dtype):
 
 # ---------------------------------------------------------------- whole models in every cutting
 LENGTHS = {"K": [40, 70, 97, 1, 33, 64, 2, 90, 340, 128, 21], "L": [97, 1, 150, 64, 31, 2, 120, 17, 65],
-           "M": [150, 64, 3, 65, 1, 200, 31, 90], "N": [40, 100, 7, 64, 130, 2, 55]}
+           "M": [150, 64, 3, 65, 1, 200, 31, 90], "N": [40, 100, 7, 64, 130, 2, 55], "P": [90, 33, 1, 140, 64, 2, 17, 120, 75, 200, 48, 100]}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
