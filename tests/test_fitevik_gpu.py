@@ -57,7 +57,7 @@ def computed(r, rt):
 
 # ---------------------------------------------------------------- each mechanism alone
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W", [52, 40, 256, 1000])
+@pytest.mark.parametrize("W", [52, 40, 37, 42, 256, 1000])
 def test_layer_norm_ahead_and_behind(dtype, W):
     """The norm as a part: of a row, of picked rows, with a delta added on the way, and as the norm of a
     sublayer's output added to the stream (which the kernel also leaves in the compute dtype)."""
