@@ -382,6 +382,26 @@ def test_single_tokens_behind_a_long_window_deal_their_keys_out():
         assert np.abs(got[n - 20:] - want).max() < 3e-2 * np.abs(want).max(), window
 
 
+def test_the_matrix_core_kernel_at_the_size_of_a_real_layer():
+    """32 heads over 8 key/value heads of 128, a window of 1,024: a prompt of 2,048 tokens whose keys are dealt out in
+    parts of 512, a portion beside it, and single tokens whose keys are dealt out in parts of 64, on the matrix cores
+    against the plain kernel (which the other tests hold against the plain implementation) with the same weights."""
+    from flambeau_amd.engine import Runtime
+    from flambeau_amd.kernels import mixed_attention
+    from flambeau_amd.parts import MIXERS
+    W, H, G, D, window, n = 128, 32, 8, 128, 1024, 2060
+    x = _x(n, W, "bfloat16", 3)
+    outs = []
+    for tuned in (True, False):
+        rt = Runtime(DEV, torch.bfloat16, 2304, tuned)
+        mixer, _ = bound_part(MIXERS, mixed_spec(W, H, G, D, D, window, D ** -0.5 * 4, 1e-5), "bfloat16", rt, seed=9, fix={"sink": lambda v: v * 8})
+        assert isinstance(mixer.kernels, mixed_attention.TunedMixedAttention) == tuned
+        outs.append([run_mixer(mixer, rt, x, cuts, page_size=16, n_pages=140) for cuts in ([2048] + [1] * 12, [700, 40, 1308] + [2] * 6)])
+    for got, want in zip(*outs):
+        err = np.abs(got - want).max(axis=1)
+        assert np.isfinite(got).all() and err.max() < 3e-2 * np.abs(want).max(), int(err.argmax())
+
+
 # ---------------------------------------------------------------- layer by layer
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", list(CONFIGS))
