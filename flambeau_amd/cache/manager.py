@@ -6,7 +6,9 @@ request, one block table (entry ``i`` = page holding tokens ``[i*ps, (i+1)*ps)``
 serves all its layers.  Pages return to the free list when a request ends, when it is
 pre-empted, and, in a windowed group, as soon as every token in them lies below the
 window of all future queries; the table keeps a hole (-1) there so that token ``t`` is
-always found at ``table[t // ps]``.
+always found at ``table[t // ps]``.  A group may also keep the first tokens of every request
+whatever its window says (``keep_first``), or, instead of a window, need only the tokens of the
+newest run of ``chunk`` positions counted from 0.
 
 Beside the pages every live request holds one *slot*: the index of its record in the
 per-request state of fixed size that layers may keep (none for attention).
@@ -63,10 +65,14 @@ class PagePool:
 @dataclass(frozen=True)
 class GroupSpec:
     """A cache group as the manager sees it: all it reads is ``window`` (newest rows still needed,
-    0 = all).  Any object with that attribute serves (``parts.base.PageGroup`` in the engine)."""
+    0 = all) and, where they exist, ``keep_first`` (rows at a request's start that stay needed) and ``chunk``
+    (instead of a window: only the newest run of ``chunk`` positions, counted from 0, is needed).  Any object with
+    ``window`` serves (``parts.base.PageGroup`` in the engine)."""
     n_kv_heads: int = 1
     head_dim: int = 1
     window: int = 0
+    keep_first: int = 0
+    chunk: int = 0
 
 
 @dataclass
@@ -161,13 +167,19 @@ class CacheManager:
                 raise CacheError(f"request {request_id!r}: advanced to {new_len} tokens beyond its pages")
         rc.n_cached = new_len
         for g, spec in enumerate(self.groups):
-            if spec.window <= 0:
+            chunk, kept = getattr(spec, "chunk", 0), getattr(spec, "keep_first", 0)
+            if spec.window > 0:
+                # the next query sits at position new_len and sees keys >= new_len - window + 1
+                first_needed = new_len - spec.window + 1
+            elif chunk > 0:
+                # ... or the keys of its own run of chunk positions
+                first_needed = new_len - new_len % chunk
+            else:
                 continue
-            # the next query sits at position new_len and sees keys >= new_len - window + 1
-            first_needed = new_len - spec.window + 1
             dead_blocks = max(0, first_needed) // self.page_size
+            kept_blocks = -(-kept // self.page_size)          # blocks with a token that stays visible are never given back
             t = rc.tables[g]
-            for b in range(rc.first_live[g], min(dead_blocks, len(t))):
+            for b in range(max(rc.first_live[g], kept_blocks), min(dead_blocks, len(t))):
                 if t[b] >= 0:
                     self.pools[g].release(t[b])
                     t[b] = -1

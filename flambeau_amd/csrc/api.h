@@ -112,6 +112,15 @@ int fl_headnorm_gate(const float* x, const float* w, const float* gate, int ldg,
 int fl_moe_route(const float* logits, int ld, int col0, int n, int E, int top, int kind, int renorm,
                  int* place, int* src_row, float* src_scale, float* pair_w, int* tiles, int max_tiles,
                  hipStream_t stream);
+// the same for a router whose choice goes by softmax + correction inside the best groups of experts and whose last
+// n_identity outputs are identity experts (E counts all outputs); weights = chosen softmax / their sum * scale
+int fl_moe_route_grouped(const float* logits, int ld, int col0, int n, int E, int n_identity, int top,
+                         const float* correction, int n_groups, int keep_groups, float scale, int* place,
+                         int* src_row, float* src_scale, float* pair_w, int* tiles, int max_tiles,
+                         hipStream_t stream);
+// y[p] = src_scale[p] * x[src_row[p]] for the sorted places of identity experts' tiles
+int fl_moe_identity(const void* x, int dtype, const int* src_row, const float* src_scale, float* y,
+                    const int* tiles, int max_tiles, int W, hipStream_t stream);
 int fl_moe_tile_rows(void);
 int fl_moe_gemm(const void* x, int dtype, const int* src_row, const float* src_scale, const void* w,
                 float* out, const int* tiles, int max_tiles, int N, int K, hipStream_t stream);
@@ -294,7 +303,7 @@ int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, int col_v, c
                    const int* tok_seq, const int* block_table, int max_blocks, void* q_out, void* cache_base,
                    int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
                    int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
-                   float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
+                   const float* q_head_gain, const float* k_head_gain, float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
                    float* row_scales, hipStream_t stream);
 
 // ---- linear recurrences with a matrix state per head (linear_scan.hip) ----
@@ -309,6 +318,18 @@ int fl_conv_prepare(const float* proj, int ld, int col0, int col_b, int col_a, c
                     const int* tok_seq, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
                     float* prep, float* gates, int n, int n_seqs, int G, int H, int D, int Dv, int taps,
                     float q_scale, float unit_eps, hipStream_t stream);
+// fl_linear_scan's delta rule with a decay per token, head and key dim (decay rows ldd wide, heads x D; beta rows ldb wide)
+int fl_linear_scan_delta_channel(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                                 const float* decay, int ldd, const float* beta, int ldb, float* state,
+                                 long slot_stride, const int* seq_q_start, const int* seq_q_len,
+                                 const int* seq_slots, float* out, int n_seqs, int H, int G, int D, int Dv,
+                                 hipStream_t stream);
+// out[t][h * D + d] = exp(-exp(a_log[h]) * softplus(a[t][col + h * D + d] + dt_bias[h * D + d]))
+int fl_channel_decay(const float* a, int ld, int col, const float* a_log, const float* dt_bias, float* out,
+                     int n, int H, int D, hipStream_t stream);
+// out[t][f] = sum_r x[t][col + r] * w[f][r]: the second factor of a projection of low rank (x float, w in dtype)
+int fl_lowrank_expand(const float* x, int ld, int col, const void* w, int dtype, float* out, int n, int N, int R,
+                      hipStream_t stream);
 int fl_rotate_scale(const float* proj, int ld, int col_a, int col_b, const float* cs, int rot, int interleaved,
                     float scale_a, float scale_b, float* out_a, float* out_b, int n, int H, int D,
                     hipStream_t stream);
@@ -342,15 +363,26 @@ int fl_forget_gates(const float* proj, int ld, int col_q, int col_f, const float
 int fl_attn_mixed_max_heads(int hd);
 int fl_attn_mixed(const void* q, void* out, const void* cache_base, int dtype, const int* positions,
                   const int* tok_seq, const int* block_table, int max_blocks, int n, int nh, int nkv, int hd,
-                  int page_size, int n_pages, float scale, int window, const float* slopes, const float* talk,
-                  const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
+                  int page_size, int n_pages, float scale, int window, int keep_first, int chunk, const float* slopes,
+                  const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
                   hipStream_t stream);
 int fl_attn_mixed_tiled_fits(int nh, int hd, int page_size);
 int fl_attn_mixed_tiled(const void* q, void* out, const void* cache_base, const int* positions, const int* block_table,
                         int max_blocks, const int* seq_q_start, const int* seq_q_len, int n_seqs, int n_tiles, int n,
-                        int nh, int nkv, int hd, int page_size, int n_pages, float scale, int window, const float* slopes,
-                        const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
+                        int nh, int nkv, int hd, int page_size, int n_pages, float scale, int window, int keep_first, int chunk,
+                        const float* slopes, const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
                         hipStream_t stream);
+
+// ---- hyper-connections: a residual stream in S copies (hyper.hip) ----
+// xs [n][S][W] float.  y given: x_t <- sum_s mix[s][t] x_s + out_w[t] * y.  in_w given: u = sum_s in_w[s] x_s (the new
+// copies) into u_out, and with a gain normed = u / sqrt(mean(u^2) + eps) * gain in out_dtype.  rows (n_rows of them):
+// the tokens that are read, one output row each (only without y).
+int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* mix, const float* out_w,
+                  const float* in_w, const int* rows, int n_rows, float* u_out, const float* gain, float eps,
+                  void* normed, int out_dtype, hipStream_t stream);
+int fl_hyper_spread(const float* x, float* xs, int n, int S, int W, hipStream_t stream);
+int fl_scaled_sum(const float* a, float ca, const float* b, float cb, float* out, long total, hipStream_t stream);
+int fl_softcap_inplace(float* x, long total, float cap, hipStream_t stream);
 
 // ---- step programs (program.hip): launches recorded once, replayed with one call ----
 typedef union FlArg { void* p; long l; int i; float f; } FlArg;

@@ -1,7 +1,8 @@
 // Softmax attention over the paged cache whose heads talk to one another before the softmax.
 //
-// For a query at position i and a key at position j of the same request, inside the window
-// (0 <= i - j < window, or every j <= i where window is 0):
+// For a query at position i and a key at position j <= i of the same request that the mask lets through
+// (window > 0: i - j < window; chunk > 0 instead: i and j in the same run of `chunk` positions counted from 0;
+// neither: every j <= i; and, whatever the rest says, every j < keep_first: the first tokens stay visible):
 //     raw_g    = scale * (q_g . k_kv(g),j) - slope_g * (i - j)            every query head g; slope may be absent
 //     score_h  = sum_g talk[h][g] * raw_g                                 the heads' scores mixed; talk may be absent
 //     weight_h = exp(score_h) / (sum over the window's j of exp(score_h) + exp(sink_h))
@@ -27,11 +28,16 @@
 
 struct AttnMixed {
     const int* positions; const int* tok_seq; const int* block_table; int max_blocks;
-    int nh; float scale; int window;
+    int nh; float scale; int window, keep_first, chunk;
     const float* slopes; const float* talk; const float* sink;
     int part_keys, n_parts;          // part_keys 0: one block takes all keys of a token and finishes it
     float* part_acc; float* part_ml; // [n][parts][nh][hd] and [n][parts][nh][2] (running maximum, sum)
 };
+
+// the first key that the window or the chunk of a query at position p lets through
+__device__ __forceinline__ int am_mask_lo(const AttnMixed& a, int p) {
+    return a.chunk > 0 ? p - p % a.chunk : a.window > 0 ? max(0, p - a.window + 1) : 0;
+}
 
 template <typename T> struct Vec8;
 template <> struct Vec8<bf16_t> {
@@ -62,7 +68,8 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
     const int token = blockIdx.x, tid = threadIdx.x;
     const int p = a.positions[token];
     const int* table = a.block_table + (size_t)a.tok_seq[token] * a.max_blocks;
-    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    const int lo = am_mask_lo(a, p);
+    const int kept = min(a.keep_first, lo);          // the keys [0, kept) are seen beside [lo, p]; the first part's block takes them
     int k0 = lo, k1 = p;
     if (a.part_keys > 0) {
         const int part = lo / a.part_keys + blockIdx.y;
@@ -95,6 +102,15 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
     for (int u = 0; u < ACC; ++u) acc[u] = 0.f;
     __syncthreads();
     const T* base_ptr = (const T*)cache.base;
+    const int main_k0 = k0, main_k1 = k1;
+    for (int range = 0; range < 2; ++range) {
+    // two runs of keys: the kept first tokens (if the mask hides what follows them), then the window's or chunk's own
+    if (range == 0) {
+        if (kept <= 0 || (a.part_keys > 0 && blockIdx.y != 0)) continue;
+        k0 = 0; k1 = kept - 1;
+    } else {
+        k0 = main_k0; k1 = main_k1;
+    }
     for (int base = (k0 / AM_CHUNK) * AM_CHUNK; base <= k1; base += AM_CHUNK) {
         // ---- the products of every head with every key of the chunk
         for (int e = tid; e < nh * AM_CHUNK; e += AM_THREADS) {
@@ -184,6 +200,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_mixed_kernel(const T* __restr
         }
         __syncthreads();
     }
+    }
     if (a.part_keys > 0) {
         float* pa = a.part_acc + ((size_t)token * a.n_parts + blockIdx.y) * nh * hd;
 #pragma unroll
@@ -245,19 +262,19 @@ extern "C" int fl_attn_mixed_max_heads(int hd) {
 
 extern "C" int fl_attn_mixed(const void* q, void* out, const void* cache_base, int dtype, const int* positions,
                              const int* tok_seq, const int* block_table, int max_blocks, int n, int nh, int nkv, int hd,
-                             int page_size, int n_pages, float scale, int window, const float* slopes, const float* talk,
-                             const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
+                             int page_size, int n_pages, float scale, int window, int keep_first, int chunk, const float* slopes,
+                             const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
                              hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_mixed: bad head counts %d/%d", nh, nkv);
     FL_CHECK(hd > 0 && hd % 8 == 0, "attn_mixed: heads are stored in multiples of 8 values, got %d", hd);
-    FL_CHECK(window >= 0, "attn_mixed: negative window");
+    FL_CHECK(window >= 0 && keep_first >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "attn_mixed: a window of %d keys, %d kept first tokens, chunks of %d", window, keep_first, chunk);
     FL_CHECK(nh <= fl_attn_mixed_max_heads(hd), "attn_mixed: %d heads of %d values are more than a block holds (%d)", nh, hd,
              fl_attn_mixed_max_heads(hd));
     FL_CHECK(part_keys >= 0 && part_keys % AM_CHUNK == 0, "attn_mixed: parts of %d keys (a multiple of %d wanted)", part_keys, AM_CHUNK);
     FL_CHECK(part_keys == 0 || (n_parts > 0 && n_parts <= 65535 && part_acc && part_ml), "attn_mixed: parts without their buffers");
     if (n == 0) return 0;
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
-    AttnMixed a{positions, tok_seq, block_table, max_blocks, nh, scale, window, slopes, talk, sink,
+    AttnMixed a{positions, tok_seq, block_table, max_blocks, nh, scale, window, keep_first, chunk, slopes, talk, sink,
                 part_keys, part_keys ? n_parts : 1, part_acc, part_ml};
     const size_t lds = 4 * ((size_t)nh * hd + 2 * nh * AM_CHUNK + (size_t)nh * nh + 4 * nh);
     dim3 grid(n, a.n_parts);
@@ -361,7 +378,8 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     const int* table = a.block_table + (size_t)seq * a.max_blocks;
     const int safe_page = table[p_last / ps];
     const bool live = safe_page >= 0 && safe_page < cache.n_pages;      // (a padding row of a fixed-size batch has no page)
-    const int lo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+    const int lo = am_mask_lo(a, p_first);             // (the first key of a row's window or chunk never falls as the rows go on)
+    const int kept = min(a.keep_first, lo);            // the keys [0, kept) are seen beside the rows' own runs; the first part's block takes them
     int k0 = lo, k1 = p_last;
     if (a.part_keys > 0) {
         const int part = lo / a.part_keys + blockIdx.y;
@@ -393,10 +411,11 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     const int rh = tid >> 4, rq = tid & 15;
     const bool row_on = rh < nh && rq < cnt;
     const int rp = p_first + rq;
-    const int r_lo = max(k0, a.window > 0 ? rp - a.window + 1 : 0), r_hi = min(k1, rp);
+    const int own_lo = am_mask_lo(a, rp);              // this row sees j in [own_lo, rp] and j < keep_first
     float rm = -INFINITY, rl = 0.f;
     // keys that every row of the tile sees: from the last row's first key to the first row's position, inside this block's part
-    const int all_lo = max(k0, a.window > 0 ? p_last - a.window + 1 : 0), all_hi = min(k1, p_first);
+    const int all_lo = max(k0, am_mask_lo(a, p_last)), all_hi = min(k1, p_first);
+    const int main_k0 = k0, main_k1 = k1;
     f32x4 o[4][DT];
 #pragma unroll
     for (int hi = 0; hi < 4; ++hi)
@@ -406,6 +425,16 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
     const int HPW = (nh + AT_WAVES - 1) / AT_WAVES;      // heads per wave, consecutive ones: at most 4
     __syncthreads();
 
+    for (int range = 0; range < 2; ++range) {
+    // two runs of keys: the kept first tokens (if the mask hides what follows them), then the rows' own
+    if (range == 0) {
+        if (kept <= 0 || (a.part_keys > 0 && blockIdx.y != 0)) continue;
+        k0 = 0; k1 = kept - 1;
+    } else {
+        k0 = main_k0; k1 = main_k1;
+    }
+    const int r_hi = min(k1, rp);
+    auto seen = [&](int j) { return j >= k0 && j <= r_hi && (j >= own_lo || j < a.keep_first); };
     for (int base = (k0 / AT_CHUNK) * AT_CHUNK; base <= k1; base += AT_CHUNK) {
         // ---- 1. raw scores: a wave takes HPW consecutive heads
         {
@@ -484,7 +513,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
         if (rh < nh) {
             u32x4* prow4 = (u32x4*)(pb + (rh * AT_ROWS + rq) * AT_P_LD);      // eight weights a store
             const float* srow = sc + rh * AT_SC_LD + rq * (AT_CHUNK + 1);
-            const bool inside = base >= all_lo && base + AT_CHUNK - 1 <= all_hi;     // (the same for the whole block)
+            const bool inside = range == 1 && base >= all_lo && base + AT_CHUNK - 1 <= all_hi;     // (the same for the whole block)
             auto pack = [](float e0, float e1) {
                 const bf16_t b0 = (bf16_t)e0, b1 = (bf16_t)e1;
                 return (unsigned)__builtin_bit_cast(unsigned short, b0) | ((unsigned)__builtin_bit_cast(unsigned short, b1) << 16);
@@ -517,7 +546,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
                 float mx = -INFINITY;
                 if (row_on)
                     for (int j = 0; j < AT_CHUNK; ++j)
-                        if (base + j >= r_lo && base + j <= r_hi) mx = fmaxf(mx, srow[j]);
+                        if (seen(base + j)) mx = fmaxf(mx, srow[j]);
                 if (mx == -INFINITY) {                                        // no key of this chunk for this row
                     for (int j8 = 0; j8 < AT_CHUNK / 8; ++j8) prow4[j8] = (u32x4){0u, 0u, 0u, 0u};
                     corr[rh * AT_ROWS + rq] = 1.f;
@@ -530,8 +559,8 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
 #pragma unroll
                         for (int j = 0; j < 8; j += 2) {
                             const int jp = base + j8 + j;
-                            const float e0 = (jp >= r_lo && jp <= r_hi) ? __expf(srow[j8 + j] - m_new) : 0.f;
-                            const float e1 = (jp + 1 >= r_lo && jp + 1 <= r_hi) ? __expf(srow[j8 + j + 1] - m_new) : 0.f;
+                            const float e0 = seen(jp) ? __expf(srow[j8 + j] - m_new) : 0.f;
+                            const float e1 = seen(jp + 1) ? __expf(srow[j8 + j + 1] - m_new) : 0.f;
                             sum += e0 + e1;
                             w[j >> 1] = pack(e0, e1);
                         }
@@ -593,6 +622,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
         }
         __syncthreads();
     }
+    }
 
     // ---- the rows' maxima and sums go to the waves that hold the outputs (or to the parts' scratch)
     float* hm = sc;
@@ -641,18 +671,19 @@ extern "C" int fl_attn_mixed_tiled_fits(int nh, int hd, int page_size) {
 // ``n_tiles``: the sum over the step's requests of ceil(rows / 16), which the caller knows from the rows per request
 extern "C" int fl_attn_mixed_tiled(const void* q, void* out, const void* cache_base, const int* positions, const int* block_table,
                                    int max_blocks, const int* seq_q_start, const int* seq_q_len, int n_seqs, int n_tiles, int n,
-                                   int nh, int nkv, int hd, int page_size, int n_pages, float scale, int window, const float* slopes,
-                                   const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc, float* part_ml,
-                                   hipStream_t stream) {
+                                   int nh, int nkv, int hd, int page_size, int n_pages, float scale, int window, int keep_first, int chunk,
+                                   const float* slopes, const float* talk, const float* sink, int part_keys, int n_parts, float* part_acc,
+                                   float* part_ml, hipStream_t stream) {
     FL_CHECK(n >= 0 && nkv > 0 && nh % nkv == 0, "attn_mixed_tiled: bad head counts %d/%d", nh, nkv);
     FL_CHECK(fl_attn_mixed_tiled_fits(nh, hd, page_size), "attn_mixed_tiled: %d heads of %d values over pages of %d are not what the kernel takes",
              nh, hd, page_size);
     FL_CHECK(window >= 0 && n_seqs >= 0 && n_tiles >= 0 && n_tiles <= n, "attn_mixed_tiled: bad window or tile count");
+    FL_CHECK(keep_first >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "attn_mixed_tiled: a window of %d keys, %d kept first tokens, chunks of %d", window, keep_first, chunk);
     FL_CHECK(part_keys >= 0 && part_keys % AT_CHUNK == 0, "attn_mixed_tiled: parts of %d keys (a multiple of %d wanted)", part_keys, AT_CHUNK);
     FL_CHECK(part_keys == 0 || (n_parts > 0 && n_parts <= 65535 && part_acc && part_ml), "attn_mixed_tiled: parts without their buffers");
     if (n == 0 || n_tiles == 0) return 0;
     PagedCache c{(void*)cache_base, nkv, page_size, hd, n_pages};
-    AttnMixed a{positions, nullptr, block_table, max_blocks, nh, scale, window, slopes, talk, sink,
+    AttnMixed a{positions, nullptr, block_table, max_blocks, nh, scale, window, keep_first, chunk, slopes, talk, sink,
                 part_keys, part_keys ? n_parts : 1, part_acc, part_ml};
     AttnTiles tl{seq_q_start, seq_q_len, n_seqs};
     const int HP = (nh + 15) & ~15;

@@ -1,0 +1,151 @@
+// Hyper-connections: a residual stream kept in S copies, and what a sublayer does to them.
+//
+// The copies of a token lie side by side, xs[t][s][i] (float).  Around a sublayer with the learned numbers
+// in[S], out[S] and mix[S][S] (indexed [from][to]):
+//     u   = sum_s in[s] x_s                      what the sublayer's norm reads
+//     x_t <- sum_s mix[s][t] x_s + out[t] * y    all copies at once from the old ones, y the sublayer's output
+// fl_hyper_step does the second line for the sublayer that has just run (if y is given) and the first for the one
+// that runs next (if `in` is given), in one pass over the copies: the new copies are written, their weighted sum u is
+// kept in float (u_out) and, if a gain is given, normed in the same kernel:
+//     normed = u / sqrt(mean(u^2) + eps) * gain      (the gain as it multiplies: one plus the stored weight, for a
+//                                                     norm whose weight is stored around zero)
+// `in` of ones and no gain gives the plain sum of the copies (what the model's last norm reads).
+// fl_hyper_spread makes the S copies of the embedding's output.  All arithmetic is float; only `normed` is stored
+// in the compute type.
+#include "common.h"
+#include "api.h"
+#include "recordable.h"
+
+#define HY_MAX_STREAMS 16
+
+struct HyperStep {
+    float* xs; int S, W;
+    const float* y;                 // [n][W] or null: nothing is written
+    const float* mix; const float* out_w;
+    const float* in_w;              // [S] or null: nothing is read
+    float* u_out;                   // [n][W] or null
+    const float* gain; float eps;   // [W] or null
+    const int* rows;                // picks the tokens that are read (one output row each), or null; only without y
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void hyper_step_kernel(HyperStep a, T* __restrict__ normed) {
+    __shared__ float coef[HY_MAX_STREAMS * HY_MAX_STREAMS + 2 * HY_MAX_STREAMS];
+    __shared__ float lds[4];
+    const int S = a.S, W = a.W;
+    float* mixs = coef;                               // [from][to]
+    float* outs = coef + HY_MAX_STREAMS * HY_MAX_STREAMS;
+    float* ins = outs + HY_MAX_STREAMS;
+    for (int e = threadIdx.x; e < S * S; e += 256) mixs[e] = a.y ? a.mix[e] : 0.f;
+    for (int e = threadIdx.x; e < S; e += 256) {
+        outs[e] = a.y ? a.out_w[e] : 0.f;
+        ins[e] = a.in_w ? a.in_w[e] : 0.f;
+    }
+    __syncthreads();
+    const int r = blockIdx.x;
+    const int t = a.rows ? a.rows[r] : r;
+    float* x = a.xs + (size_t)t * S * W;
+    const float* yr = a.y ? a.y + (size_t)t * W : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        float old[HY_MAX_STREAMS], now[HY_MAX_STREAMS];
+#pragma unroll
+        for (int s = 0; s < HY_MAX_STREAMS; ++s) old[s] = s < S ? x[(size_t)s * W + i] : 0.f;
+        float u = 0.f;
+        if (yr) {
+            const float yv = yr[i];
+#pragma unroll
+            for (int to = 0; to < HY_MAX_STREAMS; ++to) {
+                if (to >= S) break;
+                float v = 0.f;
+#pragma unroll
+                for (int s = 0; s < HY_MAX_STREAMS; ++s)
+                    if (s < S) v = fmaf(mixs[s * S + to], old[s], v);
+                now[to] = fmaf(outs[to], yv, v);
+                x[(size_t)to * W + i] = now[to];
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < HY_MAX_STREAMS; ++s) now[s] = old[s];
+        }
+        if (a.in_w) {
+#pragma unroll
+            for (int s = 0; s < HY_MAX_STREAMS; ++s)
+                if (s < S) u = fmaf(ins[s], now[s], u);
+            if (a.u_out) a.u_out[(size_t)r * W + i] = u;
+            ss = fmaf(u, u, ss);
+        }
+    }
+    if (!a.in_w || !a.gain) return;
+    ss = block_sum<4>(ss, lds);                       // (the barrier inside also orders this block's u_out stores before its reads)
+    const float inv = 1.0f / sqrtf(ss / (float)W + a.eps);
+    for (int i = threadIdx.x; i < W; i += 256)
+        normed[(size_t)r * W + i] = from_f32<T>(a.u_out[(size_t)r * W + i] * inv * a.gain[i]);
+}
+
+extern "C" int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* mix, const float* out_w,
+                             const float* in_w, const int* rows, int n_rows, float* u_out, const float* gain, float eps,
+                             void* normed, int out_dtype, hipStream_t stream) {
+    FL_CHECK(n >= 0 && S >= 1 && S <= HY_MAX_STREAMS && W > 0, "hyper_step: %d copies of %d values (at most %d copies)", S, W, HY_MAX_STREAMS);
+    FL_CHECK(!y || (mix && out_w), "hyper_step: a sublayer's output without its numbers");
+    FL_CHECK(!gain || (in_w && u_out && normed), "hyper_step: a norm needs what it reads and where it writes");
+    FL_CHECK(!rows || !y, "hyper_step: picked rows are read only");
+    const int blocks = rows ? n_rows : n;
+    if (blocks <= 0) return 0;
+    HyperStep a{xs, S, W, y, mix, out_w, in_w, u_out, gain, eps, rows};
+    if (out_dtype == FL_F32) hyper_step_kernel<float><<<blocks, 256, 0, stream>>>(a, (float*)normed);
+    else if (out_dtype == FL_BF16) hyper_step_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, (bf16_t*)normed);
+    else FL_CHECK(false, "hyper_step: unknown dtype %d", out_dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_hyper_step)
+
+// xs[t][s][:] = x[t][:] for every copy s
+__global__ __launch_bounds__(256) void hyper_spread_kernel(const float* __restrict__ x, float* __restrict__ xs, int S, int W) {
+    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= W) return;
+    const float v = x[(size_t)t * W + i];
+    for (int s = 0; s < S; ++s) xs[((size_t)t * S + s) * W + i] = v;
+}
+
+extern "C" int fl_hyper_spread(const float* x, float* xs, int n, int S, int W, hipStream_t stream) {
+    FL_CHECK(n >= 0 && S >= 1 && W > 0, "hyper_spread: bad sizes");
+    if (n == 0) return 0;
+    FL_CHECK(n <= 65535, "hyper_spread: %d rows are more than one grid takes", n);
+    hyper_spread_kernel<<<dim3(ceil_div(W, 256), n), 256, 0, stream>>>(x, xs, S, W);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_hyper_spread)
+
+// out = ca * a + cb * b, value by value (two mixers side by side, each with a factor)
+__global__ __launch_bounds__(256) void scaled_sum_kernel(const float* __restrict__ a, float ca, const float* __restrict__ b, float cb,
+                                                         float* __restrict__ out, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) out[i] = ca * a[i] + cb * b[i];
+}
+
+extern "C" int fl_scaled_sum(const float* a, float ca, const float* b, float cb, float* out, long total, hipStream_t stream) {
+    FL_CHECK(total >= 0, "scaled_sum: bad size");
+    if (total == 0) return 0;
+    scaled_sum_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(a, ca, b, cb, out, total);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_scaled_sum)
+
+// x <- cap * tanh(x / cap), value by value (a soft cap on logits)
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, long total, float cap) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int fl_softcap_inplace(float* x, long total, float cap, hipStream_t stream) {
+    FL_CHECK(total >= 0 && cap > 0.f, "softcap: bad size or cap");
+    if (total == 0) return 0;
+    softcap_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(x, total, cap);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_softcap_inplace)

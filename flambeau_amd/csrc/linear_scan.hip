@@ -36,13 +36,15 @@
 // the next run's values are asked for (into registers) before the walk over this run begins and put into
 // LDS after it, so that the trip to memory hides behind the walk.
 // MODE 0: a decay per head or per token and head, u = v; 1: the delta rule; 2: a decay per token, head AND key dim
-// (`k` holds the forget gates f; the key is 1 - f: what is forgotten makes room for what is written)
+// (`k` holds the forget gates f; the key is 1 - f: what is forgotten makes room for what is written); 3: the delta rule
+// with a decay per token, head and key dim (`chan_decay`, rows ldc wide, heads x D: S <- diag(g) S before the correction)
 template <int RPT, int MODE>
 __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ head_decay, const float* __restrict__ tok_decay, const float* __restrict__ beta, int ldg,
     float* __restrict__ state, size_t slot_stride, const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
-    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int G, int D, int Dv) {
+    const int* __restrict__ seq_slots, float* __restrict__ out, int H, int G, int D, int Dv,
+    const float* __restrict__ chan_decay = nullptr, int ldc = 0) {
     constexpr int NT = LS_GROUP * LS_COLS;
     constexpr int DP = LS_GROUP * RPT;                                // a row of q or k in LDS
     constexpr int RUN = RPT <= 8 ? 32 : RPT <= 16 ? 16 : 8;          // tokens per run
@@ -64,7 +66,8 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
     __shared__ __attribute__((aligned(16))) float qs[RUN * DP];
     __shared__ __attribute__((aligned(16))) float ks[RUN * DP];
     __shared__ float vs[RUN * LS_COLS], fs[RUN * 2];
-    float pq[PRE], pk[PRE], pv[PRE_V], pf0 = 0.f, pf1 = 0.f;
+    __shared__ __attribute__((aligned(16))) float gs[MODE == 3 ? RUN * DP : 4];
+    float pq[PRE], pk[PRE], pd[MODE == 3 ? PRE : 1], pv[PRE_V], pf0 = 0.f, pf1 = 0.f;
     auto fetch = [&](int t0) {                     // the values of the run that starts at token t0, into registers
         const int cnt = min(RUN, len - t0);
 #pragma unroll
@@ -75,6 +78,7 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
             const size_t row = (size_t)(start + t0 + (in ? tt : 0));
             pq[i] = in ? q[row * ldq + qk_head * D + d] : 0.f;
             pk[i] = in ? k[row * ldk + qk_head * D + d] : (MODE == 2 ? 1.f : 0.f);
+            if (MODE == 3) pd[i] = in ? chan_decay[row * ldc + head * D + d] : 1.f;
         }
 #pragma unroll
         for (int i = 0; i < PRE_V; ++i) {
@@ -84,8 +88,8 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
         }
         if (threadIdx.x < cnt) {
             const size_t row = (size_t)(start + t0 + threadIdx.x);
-            pf0 = tok_decay ? tok_decay[row * ldg + head] : fixed;
-            pf1 = MODE == 1 ? beta[row * ldg + head] : 1.f;
+            pf0 = (MODE != 3 && tok_decay) ? tok_decay[row * ldg + head] : fixed;
+            pf1 = (MODE == 1 || MODE == 3) ? beta[row * ldg + head] : 1.f;
         }
     };
     if (len > 0) fetch(0);
@@ -96,6 +100,7 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
         for (int i = 0; i < PRE; ++i) {
             qs[threadIdx.x + NT * i] = pq[i];
             ks[threadIdx.x + NT * i] = pk[i];
+            if (MODE == 3) gs[threadIdx.x + NT * i] = pd[i];
         }
 #pragma unroll
         for (int i = 0; i < PRE_V; ++i)
@@ -115,11 +120,13 @@ __global__ __launch_bounds__(LS_GROUP * LS_COLS) void linear_scan_kernel(
                 if (MODE == 2) {
                     S[u] *= kr[u];
                     kr[u] = 1.0f - kr[u];
+                } else if (MODE == 3) {
+                    S[u] *= gs[tt * DP + g * RPT + u];
                 } else {
                     S[u] *= decay;
                 }
             }
-            if (MODE == 1) {
+            if (MODE == 1 || MODE == 3) {
                 float seen0 = 0.f, seen1 = 0.f;                   // two chains of half the length
 #pragma unroll
                 for (int u = 0; u < RPT; u += 2) {
@@ -154,12 +161,15 @@ extern "C" int fl_linear_scan_max_dim(void) { return LS_GROUP * LS_MAX_ROWS; }
 static int linear_scan_launch(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                               const float* head_decay, const float* tok_decay, const float* beta, int ldg, float* state,
                               long slot_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_slots,
-                              float* out, int n_seqs, int H, int G, int D, int Dv, bool channel_decay, hipStream_t stream) {
+                              float* out, int n_seqs, int H, int G, int D, int Dv, bool channel_decay, hipStream_t stream,
+                              const float* chan_decay = nullptr, int ldc = 0) {
+    FL_CHECK(!chan_decay || (beta && !head_decay && !tok_decay && !channel_decay && ldc >= H * D),
+             "linear_scan: a decay per key dim under the delta rule comes with write strengths and without another decay");
     FL_CHECK(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0, "linear_scan: bad sizes");
     FL_CHECK(D <= LS_GROUP * LS_MAX_ROWS, "linear_scan: %d key dims per head, at most %d", D, LS_GROUP * LS_MAX_ROWS);
     FL_CHECK(ldq >= G * D && ldk >= G * D && ldv >= H * Dv, "linear_scan: rows narrower than their heads");
-    FL_CHECK(channel_decay ? (!head_decay && !tok_decay && !beta && H == G)
-                           : (!head_decay != !tok_decay), "linear_scan: one decay per head, or one per token and head, or one per token, head and key dim");
+    FL_CHECK(chan_decay || (channel_decay ? (!head_decay && !tok_decay && !beta && H == G)
+                                          : (!head_decay != !tok_decay)), "linear_scan: one decay per head, or one per token and head, or one per token, head and key dim");
     FL_CHECK((!tok_decay && !beta) || ldg >= H, "linear_scan: gate rows %d wide for %d heads", ldg, H);
     FL_CHECK(slot_stride >= (long)H * D * Dv, "linear_scan: a slot of %ld floats does not hold %d heads", slot_stride, H);
     if (n_seqs == 0) return 0;
@@ -169,10 +179,11 @@ static int linear_scan_launch(const float* q, int ldq, const float* k, int ldk, 
 #define FL_LS2(R, MODE)                                                                                               \
     linear_scan_kernel<R, MODE><<<grid, LS_GROUP * LS_COLS, 0, stream>>>(q, ldq, k, ldk, v, ldv, head_decay, tok_decay, beta, \
                                                                           ldg, state, (size_t)slot_stride, seq_q_start,        \
-                                                                          seq_q_len, seq_slots, out, H, G, D, Dv)
+                                                                          seq_q_len, seq_slots, out, H, G, D, Dv, chan_decay, ldc)
 #define FL_LS(R)             \
     do {                     \
-        if (channel_decay) FL_LS2(R, 2); \
+        if (chan_decay) FL_LS2(R, 3);    \
+        else if (channel_decay) FL_LS2(R, 2); \
         else if (beta) FL_LS2(R, 1);     \
         else FL_LS2(R, 0);               \
     } while (0)
@@ -205,6 +216,72 @@ extern "C" int fl_linear_scan_channel(const float* q, int ldq, const float* f, i
                               seq_q_len, seq_slots, out, n_seqs, H, H, D, Dv, true, stream);
 }
 FL_RECORDABLE(fl_linear_scan_channel)
+
+// The delta rule with a decay per token, head and key dim: S <- diag(g) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q.
+// decay: rows ldd wide, heads x D; beta: rows ldb wide, one per head.
+extern "C" int fl_linear_scan_delta_channel(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                                            const float* decay, int ldd, const float* beta, int ldb, float* state,
+                                            long slot_stride, const int* seq_q_start, const int* seq_q_len,
+                                            const int* seq_slots, float* out, int n_seqs, int H, int G, int D, int Dv,
+                                            hipStream_t stream) {
+    FL_CHECK(decay && beta, "linear_scan_delta_channel: decays and write strengths are both needed");
+    return linear_scan_launch(q, ldq, k, ldk, v, ldv, nullptr, nullptr, beta, ldb, state, slot_stride, seq_q_start,
+                              seq_q_len, seq_slots, out, n_seqs, H, G, D, Dv, false, stream, decay, ldd);
+}
+FL_RECORDABLE(fl_linear_scan_delta_channel)
+
+// g[t][h][d] = exp(-exp(A_log[h]) * softplus(a[t][col + h * D + d] + dt_bias[h * D + d])): the decays of a recurrence
+// that forgets per head and key dim
+__global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restrict__ a, int ld, int col, const float* __restrict__ a_log,
+                                                            const float* __restrict__ dt_bias, float* __restrict__ out, int H, int D) {
+    const int t = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= H * D) return;
+    const float z = a[(size_t)t * ld + col + e] + dt_bias[e];
+    const float sp = z > 20.f ? z : log1pf(expf(z));
+    out[(size_t)t * H * D + e] = expf(-expf(a_log[e / D]) * sp);
+}
+
+extern "C" int fl_channel_decay(const float* a, int ld, int col, const float* a_log, const float* dt_bias, float* out,
+                                int n, int H, int D, hipStream_t stream) {
+    FL_CHECK(n >= 0 && H > 0 && D > 0 && col >= 0 && ld >= col + H * D, "channel_decay: columns %d..%d of rows %d wide", col, col + H * D, ld);
+    if (n == 0) return 0;
+    FL_CHECK(n <= 65535, "channel_decay: %d rows are more than one grid takes", n);
+    channel_decay_kernel<<<dim3(ceil_div(H * D, 256), n), 256, 0, stream>>>(a, ld, col, a_log, dt_bias, out, H, D);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_channel_decay)
+
+// out[t][f] = sum_r x[t][col + r] * w[f][r] for a short run of r (the second factor of a projection of low rank):
+// x float rows, w in its storage type, float sums in rising order of r
+template <typename T>
+__global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __restrict__ x, int ld, int col, const T* __restrict__ w,
+                                                             float* __restrict__ out, int N, int R) {
+    extern __shared__ float xr[];
+    const int t = blockIdx.y;
+    for (int r = threadIdx.x; r < R; r += 256) xr[r] = x[(size_t)t * ld + col + r];
+    __syncthreads();
+    const int f = blockIdx.x * 256 + threadIdx.x;
+    if (f >= N) return;
+    const T* wr = w + (size_t)f * R;
+    float s = 0.f;
+    for (int r = 0; r < R; ++r) s = fmaf(xr[r], to_f32(wr[r]), s);
+    out[(size_t)t * N + f] = s;
+}
+
+extern "C" int fl_lowrank_expand(const float* x, int ld, int col, const void* w, int dtype, float* out, int n, int N, int R,
+                                 hipStream_t stream) {
+    FL_CHECK(n >= 0 && N > 0 && R > 0 && R <= 4096 && col >= 0 && ld >= col + R, "lowrank_expand: columns %d..%d of rows %d wide", col, col + R, ld);
+    if (n == 0) return 0;
+    FL_CHECK(n <= 65535, "lowrank_expand: %d rows are more than one grid takes", n);
+    dim3 grid(ceil_div(N, 256), n);
+    if (dtype == FL_F32) lowrank_expand_kernel<float><<<grid, 256, R * sizeof(float), stream>>>(x, ld, col, (const float*)w, out, N, R);
+    else if (dtype == FL_BF16) lowrank_expand_kernel<bf16_t><<<grid, 256, R * sizeof(float), stream>>>(x, ld, col, (const bf16_t*)w, out, N, R);
+    else FL_CHECK(false, "lowrank_expand: unknown dtype %d", dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_lowrank_expand)
 
 // What stands between the joined projection of a mixer with forget gates per key dim and its walk:
 // q = silu(q), f = lower + (1 - lower) * sigmoid(f + bias), both float, value by value.
@@ -256,9 +333,11 @@ __global__ __launch_bounds__(256) void conv_prepare_kernel(ConvPrepare a) {
     if (blockIdx.y == 0 && threadIdx.x < a.H) {
         const int h = threadIdx.x;
         const float* row = a.proj + (size_t)token * a.ld;
-        const float z = row[a.col_a + h] + a.dt_bias[h];
-        const float sp = z > 20.f ? z : log1pf(expf(z));
-        a.gates[(size_t)token * 2 * a.H + h] = expf(-expf(a.a_log[h]) * sp);
+        if (a.a_log) {                                   // (null: the decays are formed elsewhere, only the write strengths here)
+            const float z = row[a.col_a + h] + a.dt_bias[h];
+            const float sp = z > 20.f ? z : log1pf(expf(z));
+            a.gates[(size_t)token * 2 * a.H + h] = expf(-expf(a.a_log[h]) * sp);
+        }
         a.gates[(size_t)token * 2 * a.H + a.H + h] = 1.0f / (1.0f + expf(-row[a.col_b + h]));
     }
     const int unit = blockIdx.y * 4 + wave;
@@ -326,7 +405,7 @@ extern "C" int fl_conv_prepare(const float* proj, int ld, int col0, int col_b, i
     FL_CHECK(taps >= 1 && taps <= LS_MAX_TAPS, "conv_prepare: %d taps, at most %d", taps, LS_MAX_TAPS);
     FL_CHECK(H <= 256, "conv_prepare: %d heads, at most 256", H);
     const int C = 2 * G * D + H * Dv;
-    FL_CHECK(ld >= col0 + C && ld >= col_b + H && ld >= col_a + H, "conv_prepare: columns beyond rows %d wide", ld);
+    FL_CHECK(ld >= col0 + C && ld >= col_b + H && (!a_log || ld >= col_a + H), "conv_prepare: columns beyond rows %d wide", ld);
     FL_CHECK(slot_stride >= (long)(taps - 1) * C, "conv_prepare: a slot of %ld floats does not hold %d inputs of %d channels",
              slot_stride, taps - 1, C);
     if (n == 0) return 0;

@@ -84,8 +84,121 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
     }
 }
 
+// The picks of a router whose choice and weights differ: s = softmax(z) over all E outputs; the choice goes by
+// s + correction (correction may be null); the outputs form n_groups equal groups of neighbours, a group's score is
+// its largest choice score, and only outputs of the keep_groups best groups (the lower index among equals) can be
+// chosen; the weights are the chosen s divided by their sum (+ 1e-20) times scale.  A wave per token.
+__global__ __launch_bounds__(256) void moe_pick_grouped_kernel(const float* __restrict__ logits, int ld, int col0, int n, int E,
+                                                               int top, const float* __restrict__ correction, int n_groups,
+                                                               int keep_groups, float scale, int* __restrict__ place,
+                                                               float* __restrict__ pair_w) {
+    const int lane = threadIdx.x & 63;
+    const int nu = (E + 63) >> 6;
+    const int per = E / n_groups;
+    for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < n; t += gridDim.x * 4) {
+        const float* z = logits + (size_t)t * ld + col0;
+        float sv[MOE_MAX_EXPERTS / 64], cv[MOE_MAX_EXPERTS / 64];
+        float zmax = -INFINITY, zsum = 0.f;
+#pragma unroll
+        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+            sv[u] = (u < nu && lane + 64 * u < E) ? z[lane + 64 * u] : -INFINITY;
+            if (u < nu) zmax = fmaxf(zmax, sv[u]);
+        }
+        zmax = wave_max(zmax);
+#pragma unroll
+        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+            sv[u] = (u < nu && lane + 64 * u < E) ? expf(sv[u] - zmax) : 0.f;
+            zsum += sv[u];
+        }
+        zsum = wave_sum(zsum);
+#pragma unroll
+        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+            const int e = lane + 64 * u;
+            sv[u] = sv[u] / zsum;
+            cv[u] = (u < nu && e < E) ? sv[u] + (correction ? correction[e] : 0.f) : -INFINITY;
+        }
+        // best-of-wave over (value, index): the larger value, the lower index among equals
+        auto best_of = [&](float& bz, int& best) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float oz = __shfl_xor(bz, off, FL_WAVE);
+                const int oe = __shfl_xor(best, off, FL_WAVE);
+                if (oz > bz || (oz == bz && oe < best)) { bz = oz; best = oe; }
+            }
+        };
+        if (n_groups > 1 && keep_groups < n_groups) {
+            // A group is kept if fewer than keep_groups groups beat it (a larger score, or an equal one at a lower index).
+            // Every lane learns the scores of its own outputs' groups, then counts the groups that beat them; what lies
+            // outside the kept groups can no longer be chosen.
+            float own[MOE_MAX_EXPERTS / 64];
+            int beaten[MOE_MAX_EXPERTS / 64];
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) { own[u] = -INFINITY; beaten[u] = 0; }
+            for (int pass = 0; pass < 2; ++pass) {
+                for (int g = 0; g < n_groups; ++g) {
+                    float m = -INFINITY;
+#pragma unroll
+                    for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+                        const int e = lane + 64 * u;
+                        if (u < nu && e < E && e / per == g) m = fmaxf(m, cv[u]);
+                    }
+                    m = wave_max(m);
+#pragma unroll
+                    for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+                        const int mine = (lane + 64 * u) / per;
+                        if (pass == 0) {
+                            if (mine == g) own[u] = m;
+                        } else if (m > own[u] || (m == own[u] && g < mine)) {
+                            ++beaten[u];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
+                if (beaten[u] >= keep_groups) cv[u] = -INFINITY;
+        }
+        int chosen[MOE_MAX_TOP];
+        float w[MOE_MAX_TOP], wsum = 0.f;
+        for (int k = 0; k < top; ++k) {
+            float bz = -INFINITY;
+            int best = 0x7fffffff;
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+                const int e = lane + 64 * u;
+                if (u < nu && e < E && cv[u] > -INFINITY && (cv[u] > bz || (cv[u] == bz && e < best))) { bz = cv[u]; best = e; }
+            }
+            best_of(bz, best);
+            if (best == 0x7fffffff) {                              // (nothing is left to choose from: the lowest index not yet taken)
+                best = 0;
+                for (int e = 0; e < E; ++e) {
+                    bool taken = false;
+                    for (int u = 0; u < k; ++u) taken |= chosen[u] == e;
+                    if (!taken) { best = e; break; }
+                }
+            }
+            float sw = 0.f;
+#pragma unroll
+            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
+                if (u < nu && lane + 64 * u == best) { sw = sv[u]; cv[u] = -INFINITY; }      // taken
+            sw = wave_sum(sw);                                     // (one lane holds it)
+            chosen[k] = best;
+            w[k] = sw;
+            wsum += sw;
+        }
+        if (lane == 0) {
+            for (int k = 0; k < top; ++k) {
+                place[(size_t)t * top + k] = chosen[k];
+                pair_w[(size_t)t * top + k] = w[k] / (wsum + 1e-20f) * scale;
+            }
+        }
+    }
+}
+
 // The (token, expert) pairs that moe_pick_kernel left (place[pair] = expert) counted, sorted by expert and cut into tiles.
-__global__ __launch_bounds__(1024) void moe_route_kernel(int n, int E, int top, int* __restrict__ place,
+// Outputs E_real .. E - 1 of the router are identity experts (no matrices): their tiles carry expert -1, which the
+// products skip, and a 1 in the fourth place, which fl_moe_identity looks for.
+__global__ __launch_bounds__(1024) void moe_route_kernel(int n, int E, int E_real, int top, int* __restrict__ place,
                                                          int* __restrict__ src_row, float* __restrict__ src_scale,
                                                          const float* __restrict__ pair_w, int* __restrict__ tiles, int max_tiles) {
     __shared__ int count[MOE_MAX_EXPERTS];
@@ -99,15 +212,15 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(int n, int E, int top, 
         for (int e = 0; e < E; ++e) {
             first[e] = at;
             for (int r = 0; r < count[e] && tile < max_tiles; r += MOE_TILE, ++tile) {
-                tiles[4 * tile + 0] = e;
+                tiles[4 * tile + 0] = e < E_real ? e : -1;
                 tiles[4 * tile + 1] = at + r;
                 tiles[4 * tile + 2] = min(MOE_TILE, count[e] - r);
-                tiles[4 * tile + 3] = 0;
+                tiles[4 * tile + 3] = e < E_real ? 0 : 1;
             }
             at += count[e];
             count[e] = 0;                      // from here on: places handed out
         }
-        for (; tile < max_tiles; ++tile) {
+        for (; tile < max_tiles; ++tile) {      // (unused)
             tiles[4 * tile + 0] = -1;
             tiles[4 * tile + 1] = tiles[4 * tile + 2] = tiles[4 * tile + 3] = 0;
         }
@@ -141,11 +254,68 @@ extern "C" int fl_moe_route(const float* logits, int ld, int col0, int n, int E,
     const int pick_blocks = n < 4 * 1024 ? (n + 3) / 4 : 1024;
     moe_pick_kernel<<<pick_blocks, 256, 0, stream>>>(logits, ld, col0, n, E, top, kind, renorm, place, pair_w);
     FL_LAUNCH_CHECK();
-    moe_route_kernel<<<1, 1024, 0, stream>>>(n, E, top, place, src_row, src_scale, pair_w, tiles, max_tiles);
+    moe_route_kernel<<<1, 1024, 0, stream>>>(n, E, E, top, place, src_row, src_scale, pair_w, tiles, max_tiles);
     FL_LAUNCH_CHECK();
     return 0;
 }
 FL_RECORDABLE(fl_moe_route)
+
+// fl_moe_route for a router with a correction of the choice, groups of experts and identity experts (see
+// moe_pick_grouped_kernel).  E counts all the router's outputs, the last n_identity of which are identity experts.
+extern "C" int fl_moe_route_grouped(const float* logits, int ld, int col0, int n, int E, int n_identity, int top,
+                                    const float* correction, int n_groups, int keep_groups, float scale, int* place,
+                                    int* src_row, float* src_scale, float* pair_w, int* tiles, int max_tiles,
+                                    hipStream_t stream) {
+    FL_CHECK(n >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= MOE_MAX_TOP && top <= E,
+             "moe_route_grouped: %d of %d experts (at most %d of %d)", top, E, MOE_MAX_TOP, MOE_MAX_EXPERTS);
+    FL_CHECK(n_identity >= 0 && n_identity < E, "moe_route_grouped: %d identity experts among %d outputs", n_identity, E);
+    FL_CHECK(n_groups >= 1 && E % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups && keep_groups <= MOE_MAX_TOP &&
+             keep_groups * (E / n_groups) >= top, "moe_route_grouped: %d of %d groups over %d outputs cannot give %d choices",
+             keep_groups, n_groups, E, top);
+    FL_CHECK(ld >= col0 + E && col0 >= 0, "moe_route_grouped: columns %d..%d of rows %d wide", col0, col0 + E, ld);
+    {
+        const long pairs = (long)n * top;
+        FL_CHECK((long)max_tiles >= pairs / MOE_TILE + (pairs < E ? pairs : E), "moe_route_grouped: %d tiles cannot hold %ld rows of %d experts", max_tiles, pairs, E);
+    }
+    if (n == 0) return 0;
+    const int pick_blocks = n < 4 * 1024 ? (n + 3) / 4 : 1024;
+    moe_pick_grouped_kernel<<<pick_blocks, 256, 0, stream>>>(logits, ld, col0, n, E, top, correction, n_groups, keep_groups, scale,
+                                                             place, pair_w);
+    FL_LAUNCH_CHECK();
+    moe_route_kernel<<<1, 1024, 0, stream>>>(n, E, E - n_identity, top, place, src_row, src_scale, pair_w, tiles, max_tiles);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_moe_route_grouped)
+
+// The rows of identity experts: y[p] = scale[p] * x[src[p]] for the places p of every tile that fl_moe_route_grouped
+// marked as an identity expert's.
+template <typename TIn>
+__global__ __launch_bounds__(256) void moe_identity_kernel(const TIn* __restrict__ x, const int* __restrict__ src_row,
+                                                           const float* __restrict__ src_scale, float* __restrict__ y,
+                                                           const int* __restrict__ tiles, int W) {
+    if (tiles[4 * blockIdx.y + 3] != 1) return;
+    const int p0 = tiles[4 * blockIdx.y + 1], M = tiles[4 * blockIdx.y + 2];
+    for (int r = 0; r < M; ++r) {
+        const TIn* xr = x + (size_t)src_row[p0 + r] * W;
+        const float f = src_scale[p0 + r];
+        for (int c = blockIdx.x * 256 + threadIdx.x; c < W; c += 256 * gridDim.x) y[(size_t)(p0 + r) * W + c] = f * to_f32(xr[c]);
+    }
+}
+
+extern "C" int fl_moe_identity(const void* x, int dtype, const int* src_row, const float* src_scale, float* y,
+                               const int* tiles, int max_tiles, int W, hipStream_t stream) {
+    FL_CHECK(max_tiles >= 0 && W > 0 && src_row && src_scale, "moe_identity: bad sizes or no rows");
+    if (max_tiles == 0) return 0;
+    FL_CHECK(max_tiles <= 65535, "moe_identity: %d row tiles are more than one grid takes", max_tiles);
+    dim3 grid(min(ceil_div(W, 256), 16), max_tiles);
+    if (dtype == FL_F32) moe_identity_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, src_row, src_scale, y, tiles, W);
+    else if (dtype == FL_BF16) moe_identity_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, src_row, src_scale, y, tiles, W);
+    else FL_CHECK(false, "moe_identity: unknown dtype %d", dtype);
+    FL_LAUNCH_CHECK();
+    return 0;
+}
+FL_RECORDABLE(fl_moe_identity)
 
 // The plain product (64 x 64 tile, 4 x 4 per thread, k in steps of 16, the steps' sums added with a
 // compensated addition) over the rows of one tile of one expert.  src_row / src_scale may be null (the

@@ -4,7 +4,8 @@
 //     (x / sqrt(mean(x^2) + eps) * w over all heads at once), or none;
 //   * rotation of the first `rot` dims of every head from the step's table of cosines and sines, pairs
 //     (i, i + rot/2) ("half") or (2i, 2i + 1) ("interleaved");
-//   * every head of q and k divided by its root mean square after rotation (no gain), or not;
+//   * every head of q and k divided by its root mean square after rotation, with no gain or with a gain per
+//     head dim that all heads of q (of k) share, or not;
 //   * values blended with those an earlier layer made for the same token,
 //     v <- (1 - lambda) v + lambda v_first, or kept as that first layer's for later ones;
 //   * q stored for the attention kernels, k and v stored into the paged cache at the token's position.
@@ -23,6 +24,7 @@ struct QkvPrepare {
     int nh, D, Dv, hdp;
     int rot, interleaved; const float2* cs;
     const float* qnorm_w; const float* knorm_w; int head_norm; float eps;
+    const float* q_head_gain; const float* k_head_gain;   // [D] each, or null: the gain behind the heads' own norm
     float* v_first; int vmix_mode; const float* lambda;
     int write_cache;
     float* row_scales;          // [n][2]: 1 / rms of every token's q and k projection, made by a kernel of its own (or null)
@@ -102,8 +104,9 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
         }
         if (a.head_norm) {
             const float f = 1.0f / sqrtf(wave_sum(ss) / (float)D + a.eps);
+            const float* hg = is_q ? a.q_head_gain : a.k_head_gain;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) r[j] *= f;
+            for (int j = 0; j < 4; ++j) r[j] *= (hg && lane + 64 * j < D) ? f * hg[lane + 64 * j] : f;
         }
         if (is_q) {
             T* dst = q_out + ((size_t)token * nh + h) * hdp;
@@ -136,7 +139,7 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
                               const int* tok_seq, const int* block_table, int max_blocks, void* q_out, void* cache_base,
                               int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
                               int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
-                              float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
+                              const float* q_head_gain, const float* k_head_gain, float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
                               float* row_scales, hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && D > 0 && Dv > 0 && page_size > 0, "qkv_prepare: bad sizes");
     FL_CHECK(hdp >= D && hdp >= Dv && hdp <= 256, "qkv_prepare: heads of %d and %d values stored %d wide (at most 256)", D, Dv, hdp);
@@ -145,11 +148,12 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
     FL_CHECK(ld >= col_q + nh * D && (col_k < 0 || (ld >= col_k + nkv * D && ld >= col_v + nkv * Dv)), "qkv_prepare: columns beyond rows %d wide", ld);
     FL_CHECK(col_k >= 0 || !write_cache, "qkv_prepare: a projection of queries alone writes no cache");
     FL_CHECK(col_k < 0 ? !knorm_w : !qnorm_w == !knorm_w, "qkv_prepare: the norm over the projection needs both gains");
+    FL_CHECK(head_norm || (!q_head_gain && !k_head_gain), "qkv_prepare: a gain per head dim without the heads' norm");
     FL_CHECK(vmix_mode >= 0 && vmix_mode <= 2 && (vmix_mode == 0 || v_first) && (vmix_mode != 2 || lambda),
              "qkv_prepare: value blending %d without its buffers", vmix_mode);
     if (n == 0) return 0;
     QkvPrepare a{proj, ld, col_q, col_k, col_v, positions, tok_seq, block_table, max_blocks, nh, D, Dv, hdp,
-                 rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, v_first, vmix_mode, lambda, write_cache,
+                 rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, q_head_gain, k_head_gain, v_first, vmix_mode, lambda, write_cache,
                  (qnorm_w && n > QKV_FEW_TOKENS) ? row_scales : nullptr};
     PagedCache c{cache_base, nkv, page_size, hdp, n_pages};
     dim3 grid(n, ceil_div(nh + (col_k >= 0 ? nkv : 0), 4));

@@ -25,13 +25,16 @@ class PlainMixedAttention:
         """What the kernels decide from the contexts' lengths (part of a recorded step's key)."""
         return 0
 
-    def attention(self, q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink):
-        return ops.attn_mixed(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, slopes, talk, sink)
+    def attention(self, q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink, keep_first=0, chunk=0):
+        return ops.attn_mixed(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, slopes, talk, sink,
+                              keep_first=keep_first, chunk=chunk)
 
 
 class TunedMixedAttention(PlainMixedAttention):
     def signature(self, batch, window: int):
-        """``(keys per part, parts)`` a tile's keys are dealt out to; ``(0, 0)``: one block finishes a tile."""
+        """``(keys per part, parts)`` a tile's keys are dealt out to; ``(0, 0)``: one block finishes a tile.  ``window``:
+        how far back a row's own run of keys can reach (its window, or the length of its chunk of positions; 0: to
+        the start).  Kept first tokens are not dealt out: the first part's block takes them."""
         ctx = batch.ctx_bound or batch.max_ctx_len
         keys = min(window + TILE_ROWS - 1, ctx) if window else ctx          # (what the rows of a tile see together)
         if batch.n_tokens <= FEW_ROWS:
@@ -45,8 +48,8 @@ class TunedMixedAttention(PlainMixedAttention):
         parts = (keys - 1) // part_keys + 2          # (a run of keys may begin anywhere inside its first part)
         return (part_keys, 1 << (parts - 1).bit_length())
 
-    def attention(self, q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink):
-        part_keys, parts = self.signature(step.host, window)
+    def attention(self, q, out, kv, step, table, n_heads, scale, window, slopes, talk, sink, keep_first=0, chunk=0):
+        part_keys, parts = self.signature(step.host, window or chunk)
         n, rt = q.shape[0], self.rt
         split = {}
         if parts:
@@ -56,8 +59,9 @@ class TunedMixedAttention(PlainMixedAttention):
         if kv.pool.dtype == torch.bfloat16 and ops.attn_mixed_tiled_fits(n_heads, kv.head_dim, kv.page_size):
             n_tiles = sum(-(-rows // TILE_ROWS) for rows in step.host.q_lens)
             return ops.attn_mixed_tiled(q, out, kv, step.positions, table, step.seq_q_start, step.seq_q_len, n_tiles, n_heads, scale,
-                                        window, slopes, talk, sink, **split)
-        return ops.attn_mixed(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, slopes, talk, sink, **split)
+                                        window, slopes, talk, sink, keep_first=keep_first, chunk=chunk, **split)
+        return ops.attn_mixed(q, out, kv, step.positions, step.tok_seq, table, n_heads, scale, window, slopes, talk, sink,
+                              keep_first=keep_first, chunk=chunk, **split)
 
 
 register_kernel_set("mixed_heads_attention", PlainMixedAttention, TunedMixedAttention)

@@ -437,7 +437,7 @@ def moe_max_tiles(n_pairs: int, n_experts: int) -> int:
     return n_pairs // moe_tile_rows() + min(n_pairs, n_experts)
 
 
-ROUTER_SCORINGS = {"sigmoid": 0, "softmax": 1, "softmax_chosen": 2}
+ROUTER_SCORINGS = {"sigmoid": 0, "softmax": 1, "softmax_chosen": 2, "softmax_grouped": 3}     # (the last has a launch function of its own)
 
 
 def moe_route(logits, col0, n_experts, top, place, src_row, src_scale, pair_w, tiles, scoring="sigmoid", renormalise=False):
@@ -569,11 +569,12 @@ def heads_gate(x, head_stride, gate, gate_col0, kind, out, n_heads):
 
 def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads, dim, vdim, rotated_dims,
                 interleaved, table, q_gain, k_gain, head_norm, eps, v_first=None, value_mix: int = 0, mix=None, write_cache=True,
-                row_scales=None):
+                row_scales=None, q_head_gain=None, k_head_gain=None):
     """From the float32 rows of a joined projection (q, k, v at the columns ``cols``) to the rotated, normed
     queries in ``q_out`` and the token's keys and values in the cache, heads stored ``cache.head_dim`` wide.
     ``q_gain`` / ``k_gain``: gains of a norm over the whole projection of q and of k (before rotation);
-    ``head_norm``: every head divided by its root mean square after rotation; ``value_mix``: 1 keeps the
+    ``head_norm``: every head divided by its root mean square after rotation, times ``q_head_gain`` / ``k_head_gain``
+    (float32 ``[dim]``, one gain per head dim that all heads share) where given; ``value_mix``: 1 keeps the
     values in ``v_first``, 2 blends them with it by the device scalar ``mix``; ``row_scales``: float32 ``[n, 2]`` of
     scratch for the norm over the projection (a step of many tokens forms its sums in a kernel of their own)."""
     n, ld = proj.shape
@@ -590,7 +591,9 @@ def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: Paged
          _check(table, "qkv_prepare.table", torch.float32, (n, half, 2)) if rotated_dims else None,
          _check(q_gain, "qkv_prepare.q_gain", torch.float32, (n_heads * dim,)) if q_gain is not None else None,
          _check(k_gain, "qkv_prepare.k_gain", torch.float32, (nkv * dim,)) if k_gain is not None else None,
-         int(bool(head_norm)), float(eps),
+         int(bool(head_norm)),
+         _check(q_head_gain, "qkv_prepare.q_head_gain", torch.float32, (dim,)) if q_head_gain is not None else None,
+         _check(k_head_gain, "qkv_prepare.k_head_gain", torch.float32, (dim,)) if k_head_gain is not None else None, float(eps),
          _check(v_first, "qkv_prepare.v_first", torch.float32, (n, nkv * vdim)) if v_first is not None else None, int(value_mix),
          _check(mix, "qkv_prepare.mix", torch.float32) if mix is not None else None, int(bool(write_cache)),
          _check(row_scales, "qkv_prepare.row_scales", torch.float32, (n, 2)) if row_scales is not None else None, stream_handle())
@@ -608,13 +611,15 @@ def conv_max_taps() -> int:
 
 
 def linear_scan(q, k, v, state, seq_q_start, seq_q_len, seq_slots, out, n_heads, n_qk_heads, dim, vdim,
-                head_decay=None, token_gates=None, channel_decay: bool = False):
+                head_decay=None, token_gates=None, channel_decay: bool = False, key_decay=None):
     """The recurrence S <- g S + k u^T, o = S^T q over the step's tokens, request by request, from and into
     the first ``heads * dim * vdim`` floats of every slot's record in ``state`` ``[slots, floats]``.
     ``q``, ``k`` float32 ``[n, n_qk_heads * dim]`` (views of wider rows are taken with their row stride),
     ``v`` ``[n, n_heads * vdim]``.  ``head_decay`` float32 ``[heads]``: a fixed g per head and u = v;
     ``token_gates`` float32 ``[n, 2 * heads]`` (g, then beta): the delta rule, u = beta (v - S^T k).
-    ``channel_decay``: ``k`` holds a forget gate f per token, head and key dim, S <- diag(f) S + (1 - f) v^T."""
+    ``channel_decay``: ``k`` holds a forget gate f per token, head and key dim, S <- diag(f) S + (1 - f) v^T.
+    ``key_decay`` float32 ``[n, heads * dim]`` beside ``token_gates``: the delta rule with a decay per token, head and
+    key dim, S <- diag(g) S before the correction (the decays of ``token_gates`` are then not read)."""
     n = out.shape[0]
     S = seq_q_start.shape[0]
     if state.dim() != 2 or not state.is_contiguous():
@@ -632,6 +637,17 @@ def linear_scan(q, k, v, state, seq_q_start, seq_q_len, seq_slots, out, n_heads,
              _check(seq_q_start, "linear_scan.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "linear_scan.seq_q_len", torch.int32, (S,)),
              _check(seq_slots, "linear_scan.seq_slots", torch.int32, (S,)), _check(out, "linear_scan.out", torch.float32, (n, n_heads * vdim)),
              S, int(n_heads), int(dim), int(vdim), stream_handle())
+        return out
+    if key_decay is not None:
+        if token_gates is None or head_decay is not None:
+            raise KernelError("linear_scan: decays per key dim under the delta rule come with the gates per token (their write strengths)")
+        pg = _check(token_gates, "linear_scan.gates", torch.float32, (n, 2 * n_heads))
+        call("fl_linear_scan_delta_channel", pq, ldq, pk, ldk, pv, ldv,
+             _check(key_decay, "linear_scan.key_decay", torch.float32, (n, n_heads * dim)), n_heads * dim, pg + 4 * n_heads, 2 * n_heads,
+             _check(state, "linear_scan.state", torch.float32), state.shape[1],
+             _check(seq_q_start, "linear_scan.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "linear_scan.seq_q_len", torch.int32, (S,)),
+             _check(seq_slots, "linear_scan.seq_slots", torch.int32, (S,)), _check(out, "linear_scan.out", torch.float32, (n, n_heads * vdim)),
+             S, int(n_heads), int(n_qk_heads), int(dim), int(vdim), stream_handle())
         return out
     if (head_decay is None) == (token_gates is None):
         raise KernelError("linear_scan: a decay per head or gates per token, one of the two")
@@ -658,8 +674,9 @@ def conv_prepare(proj, col0, col_b, col_a, conv_w, a_log, dt_bias, state, conv_a
     if state.dim() != 2 or not state.is_contiguous() or state.shape[1] < conv_at + (taps - 1) * C:
         raise KernelError(f"conv_prepare.state: shape {tuple(state.shape)} does not hold {taps - 1} x {C} floats at {conv_at}")
     call("fl_conv_prepare", _check(proj, "conv_prepare.proj", torch.float32), ld, int(col0), int(col_b), int(col_a),
-         _check(conv_w, "conv_prepare.conv_w", torch.float32, (C, taps)), _check(a_log, "conv_prepare.a_log", torch.float32, (n_heads,)),
-         _check(dt_bias, "conv_prepare.dt_bias", torch.float32, (n_heads,)),
+         _check(conv_w, "conv_prepare.conv_w", torch.float32, (C, taps)),
+         _check(a_log, "conv_prepare.a_log", torch.float32, (n_heads,)) if a_log is not None else None,       # (None: the decays are formed elsewhere)
+         _check(dt_bias, "conv_prepare.dt_bias", torch.float32, (n_heads,)) if a_log is not None else None,
          _check(state, "conv_prepare.state", torch.float32) + 4 * int(conv_at), state.shape[1],
          _check(tok_seq, "conv_prepare.tok_seq", torch.int32, (n,)), _check(seq_q_start, "conv_prepare.seq_q_start", torch.int32, (S,)),
          _check(seq_q_len, "conv_prepare.seq_q_len", torch.int32, (S,)), _check(seq_slots, "conv_prepare.seq_slots", torch.int32, (S,)),
@@ -752,10 +769,13 @@ def attn_mixed_max_heads(head_dim: int) -> int:
 
 
 def attn_mixed(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, n_heads, scale, window,
-               slopes=None, talk=None, sink=None, part_keys: int = 0, n_parts: int = 1, part_acc=None, part_ml=None):
+               slopes=None, talk=None, sink=None, part_keys: int = 0, n_parts: int = 1, part_acc=None, part_ml=None,
+               keep_first: int = 0, chunk: int = 0):
     """Attention over the paged cache with ``slopes[g] * (i - j)`` taken off the scores, the heads' scores mixed by
     ``talk`` ``[H, H]`` and ``exp(sink[h])`` in the denominator (each optional).  ``part_keys`` > 0: every
-    token's keys are dealt out to ``n_parts`` blocks; ``part_acc`` / ``part_ml`` float32 scratch for them."""
+    token's keys are dealt out to ``n_parts`` blocks; ``part_acc`` / ``part_ml`` float32 scratch for them.
+    The mask: ``window`` newest keys, or (``chunk`` > 0 instead) the keys of the query's own run of ``chunk`` positions
+    counted from 0, or all; and always the first ``keep_first`` keys."""
     n = q.shape[0]
     hd = cache.head_dim
     dt = cache.pool.dtype
@@ -767,7 +787,7 @@ def attn_mixed(q, out, cache: PagedLayerCache, positions, tok_seq, block_table, 
          _check(cache.pool, "attn_mixed.cache"), dtype_code(dt), _check(positions, "attn_mixed.positions", torch.int32, (n,)),
          _check(tok_seq, "attn_mixed.tok_seq", torch.int32, (n,)),
          _check(block_table, "attn_mixed.block_table", torch.int32, (None, None)), block_table.shape[1],
-         n, int(n_heads), cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window),
+         n, int(n_heads), cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window), int(keep_first), int(chunk),
          f(slopes, "slopes", (n_heads,)), f(talk, "talk", (n_heads, n_heads)), f(sink, "sink", (n_heads,)),
          int(part_keys), int(n_parts), f(part_acc, "part_acc", None), f(part_ml, "part_ml", None), stream_handle())
     return out
@@ -780,7 +800,8 @@ def attn_mixed_tiled_fits(n_heads: int, head_dim: int, page_size: int) -> bool:
 
 
 def attn_mixed_tiled(q, out, cache: PagedLayerCache, positions, block_table, seq_q_start, seq_q_len, n_tiles, n_heads, scale, window,
-                     slopes=None, talk=None, sink=None, part_keys: int = 0, n_parts: int = 1, part_acc=None, part_ml=None):
+                     slopes=None, talk=None, sink=None, part_keys: int = 0, n_parts: int = 1, part_acc=None, part_ml=None,
+                     keep_first: int = 0, chunk: int = 0):
     """``attn_mixed`` on the matrix cores: blocks take tiles of 16 rows of one request; ``n_tiles`` is the sum over
     the requests of ceil(rows / 16), ``seq_q_start`` / ``seq_q_len`` the first row and the rows of every request."""
     n = q.shape[0]
@@ -798,6 +819,93 @@ def attn_mixed_tiled(q, out, cache: PagedLayerCache, positions, block_table, seq
          _check(block_table, "attn_mixed_tiled.block_table", torch.int32, (None, None)), block_table.shape[1],
          _check(seq_q_start, "attn_mixed_tiled.seq_q_start", torch.int32, (S,)), _check(seq_q_len, "attn_mixed_tiled.seq_q_len", torch.int32, (S,)),
          S, int(n_tiles), n, int(n_heads), cache.n_kv_heads, hd, cache.page_size, cache.n_pages, float(scale), int(window),
-         f(slopes, "slopes", (n_heads,)), f(talk, "talk", (n_heads, n_heads)), f(sink, "sink", (n_heads,)),
+         int(keep_first), int(chunk), f(slopes, "slopes", (n_heads,)), f(talk, "talk", (n_heads, n_heads)), f(sink, "sink", (n_heads,)),
          int(part_keys), int(n_parts), f(part_acc, "part_acc", None), f(part_ml, "part_ml", None), stream_handle())
     return out
+
+
+# ---------------------------------------------------------------- hyper-connections, decays per key dim, routers with groups
+def channel_decay(a, col, a_log, dt_bias, out, n_heads, dim):
+    """``out[t, h * dim + d] = exp(-exp(a_log[h]) * softplus(a[t, col + h * dim + d] + dt_bias[h * dim + d]))``."""
+    n, ld = a.shape
+    call("fl_channel_decay", _check(a, "channel_decay.a", torch.float32), ld, int(col),
+         _check(a_log, "channel_decay.a_log", torch.float32, (n_heads,)), _check(dt_bias, "channel_decay.dt_bias", torch.float32, (n_heads * dim,)),
+         _check(out, "channel_decay.out", torch.float32, (n, n_heads * dim)), n, int(n_heads), int(dim), stream_handle())
+    return out
+
+
+def lowrank_expand(x, col, w, out):
+    """``out[t] = w @ x[t, col : col + rank]``: the second factor of a projection of low rank; ``x`` float32 rows (the
+    first factor's products, not rounded), ``w`` ``[features, rank]`` in its storage dtype, ``out`` float32."""
+    n, ld = x.shape
+    N, R = w.shape
+    call("fl_lowrank_expand", _check(x, "lowrank_expand.x", torch.float32), ld, int(col), _check(w, "lowrank_expand.w"), dtype_code(w.dtype),
+         _check(out, "lowrank_expand.out", torch.float32, (n, N)), n, N, R, stream_handle())
+    return out
+
+
+def moe_route_grouped(logits, col0, n_outputs, n_identity, top, correction, n_groups, keep_groups, scale, place, src_row, src_scale,
+                      pair_w, tiles):
+    """``moe_route`` for a router that scores by a softmax over all its ``n_outputs`` outputs (the last ``n_identity`` of
+    them identity experts), chooses by score + ``correction`` inside the ``keep_groups`` best of ``n_groups`` groups of
+    neighbours, and weights the chosen by their scores over their sum, times ``scale``."""
+    n, ld = logits.shape
+    P_ = n * top
+    call("fl_moe_route_grouped", _check(logits, "moe_route.logits", torch.float32), ld, int(col0), n, int(n_outputs), int(n_identity), int(top),
+         _check(correction, "moe_route.correction", torch.float32, (n_outputs,)) if correction is not None else None,
+         int(n_groups), int(keep_groups), float(scale),
+         _check(place, "moe_route.place", torch.int32, (P_,)), _check(src_row, "moe_route.src_row", torch.int32, (P_,)),
+         _check(src_scale, "moe_route.src_scale", torch.float32, (P_,)), _check(pair_w, "moe_route.pair_w", torch.float32, (P_,)),
+         _check(tiles, "moe_route.tiles", torch.int32, (None, 4)), tiles.shape[0], stream_handle())
+
+
+def moe_identity(x, src_row, src_scale, y, tiles):
+    """``y[p] = src_scale[p] * x[src_row[p]]`` for the sorted places of the identity experts' tiles."""
+    P_, W = y.shape
+    call("fl_moe_identity", _check(x, "moe_identity.x", None, (None, W)), dtype_code(x.dtype),
+         _check(src_row, "moe_identity.src_row", torch.int32, (P_,)), _check(src_scale, "moe_identity.src_scale", torch.float32, (P_,)),
+         _check(y, "moe_identity.y", torch.float32), _check(tiles, "moe_identity.tiles", torch.int32, (None, 4)), tiles.shape[0], W,
+         stream_handle())
+    return y
+
+
+HYPER_MAX_STREAMS = 16     # copies of a residual stream that the kernels of hyper-connections take
+
+
+def hyper_spread(x, xs, n_streams):
+    """``xs[t, s] = x[t]`` for every copy ``s``: the copies of a stream as the embedding leaves it."""
+    n, W = x.shape
+    call("fl_hyper_spread", _check(x, "hyper_spread.x", torch.float32), _check(xs, "hyper_spread.xs", torch.float32, (n, n_streams * W)),
+         n, int(n_streams), W, stream_handle())
+    return xs
+
+
+def hyper_step(xs, n_streams, y=None, mix=None, out_w=None, in_w=None, u_out=None, gain=None, eps=0.0, normed=None, rows=None):
+    """One pass over the copies ``xs`` float32 ``[n, S * W]`` of a stream.  With ``y`` (float32 ``[n, W]``, a sublayer's
+    output): x_t <- sum_s mix[s, t] x_s + out_w[t] y.  With ``in_w``: u = sum_s in_w[s] x_s of the new copies into ``u_out``
+    and, with ``gain``, ``normed = u / sqrt(mean(u^2) + eps) * gain``.  ``rows`` (int32) picks the tokens that are read."""
+    n, SW = xs.shape
+    S = int(n_streams)
+    W = SW // S
+    f = lambda t, name, shape: _check(t, "hyper_step." + name, torch.float32, shape) if t is not None else None
+    n_rows = rows.shape[0] if rows is not None else n
+    call("fl_hyper_step", _check(xs, "hyper_step.xs", torch.float32), n, S, W, f(y, "y", (n, W)), f(mix, "mix", (S, S)),
+         f(out_w, "out", (S,)), f(in_w, "in", (S,)), _check(rows, "hyper_step.rows", torch.int32) if rows is not None else None, n_rows,
+         f(u_out, "u", (n_rows, W)), f(gain, "gain", (W,)), float(eps),
+         _check(normed, "hyper_step.normed", None, (n_rows, W)) if normed is not None else None,
+         dtype_code(normed.dtype) if normed is not None else 0, stream_handle())
+
+
+def scaled_sum(a, factor_a, b, factor_b, out):
+    """``out = factor_a * a + factor_b * b`` (float32, equal shapes)."""
+    if a.shape != b.shape or a.shape != out.shape:
+        raise KernelError(f"scaled_sum: shapes {tuple(a.shape)}, {tuple(b.shape)}, {tuple(out.shape)} differ")
+    call("fl_scaled_sum", _check(a, "scaled_sum.a", torch.float32), float(factor_a), _check(b, "scaled_sum.b", torch.float32), float(factor_b),
+         _check(out, "scaled_sum.out", torch.float32), a.numel(), stream_handle())
+    return out
+
+
+def softcap_inplace(x, cap: float):
+    """``x <- cap * tanh(x / cap)`` (float32)."""
+    call("fl_softcap_inplace", _check(x, "softcap.x", torch.float32), x.numel(), float(cap), stream_handle())
+    return x

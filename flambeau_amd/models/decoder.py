@@ -17,6 +17,7 @@ import torch
 from ..kernels import ops
 from ..kernels.library import suspended
 from ..parts import BLOCKS, EMBEDDINGS, HEADS, NORMS, PartSpec, ResidualStream
+from ..parts.block import HyperStream
 
 
 @dataclass
@@ -49,6 +50,7 @@ class ModelSpec:
     eos_token_ids: tuple = ()         # every id that ends a sequence (eos_token_id is the first)
     ignored_tensors: tuple = ()       # name patterns (fnmatch) of tensors a file may hold and the model does not read
     keeps_embedding: bool = False     # a copy of the embedding's output stays in StepState.scratch["embedding_output"] for blocks that read it
+    residual_streams: int | None = None   # the residual stream is kept in this many copies (hyper-connections; blocks of kind "hyper_prenorm"); None: one stream, plain sums
 
 
 SMALL_STEP = 16      # up to this many rows the output head runs on every row of a step
@@ -64,6 +66,8 @@ class DecoderModel:
         self.final_norm = NORMS.create(spec.final_norm)
         self.head = HEADS.create(spec.head or PartSpec("linear_head", dict(sizes, tied=spec.tied_head)))
         self._signature_mixers = None
+        self._stream_ones = (torch.ones(spec.residual_streams, dtype=torch.float32, device=rt.device)
+                             if spec.residual_streams is not None else None)
         self._recorded_blocks = None        # per block: can its launches be recorded?
         seen: dict = {}
         self._visits = []                   # per run-order entry: how many earlier entries ran the same layer
@@ -201,13 +205,18 @@ class DecoderModel:
         if self.spec.keeps_embedding:
             step.scratch["embedding_output"] = self.embedding.forward(
                 step.tokens, rt.buffer("embedding_output", step.n_tokens, self.spec.hidden_size, torch.float32), **with_step)
-        stream = ResidualStream(resid, rt)
+        if self.spec.residual_streams is not None:
+            stream = HyperStream(resid, rt, self.spec.residual_streams, self._stream_ones)
+        else:
+            stream = ResidualStream(resid, rt)
         if self._recorded_blocks is None:
             self._recorded_blocks = [self._part_replayable(b) for b in self.blocks]
         for i, e in enumerate(self.spec.run_order):
             block = self.blocks[e.layer]
             step.visit = self._visits[i]
             if step.recorder is not None and not self._recorded_blocks[e.layer]:
+                if self.spec.residual_streams is not None:
+                    raise NotImplementedError("a block that cannot be recorded in a model whose residual stream is kept in several copies")
                 # A block that cannot be replayed ends the recorded stretch: when the step is replayed it
                 # runs again with that step's metadata.  Whatever it allocates lies elsewhere then, so
                 # all that passes between it and the recorded stretches is the residual stream itself:

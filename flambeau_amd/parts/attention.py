@@ -117,7 +117,8 @@ class NormedGQAAttention(PagedGQAAttention):
       attention kernels of one head size serve both;
     * ``qk_norm``: ``"projection"``: q (and k) divided by the root mean square over ALL its heads at once,
       times a gain per value, before rotation; ``"head"``: every head of q and k divided by its own root
-      mean square after rotation, no gain; ``None``;
+      mean square after rotation, no gain; ``"head_gain"``: the same with a gain per head dim that all heads of q
+      (of k) share; ``None``;
     * ``position``: any encoding that offers a table of cosines and sines and a ``layout`` (``half`` or
       ``interleaved``), or ``none``;
     * ``softcap``: score <- softcap * tanh(score / softcap) before the softmax;
@@ -140,8 +141,8 @@ class NormedGQAAttention(PagedGQAAttention):
         value_dim = head_dim if value_dim is None else value_dim
         self.value_dim = value_dim
         self.stored_dim = -(-max(head_dim, value_dim) // 8) * 8
-        if qk_norm not in (None, "projection", "head"):
-            raise ValueError(f"normed_gqa_attention: qk_norm must be 'projection', 'head' or None, got {qk_norm!r}")
+        if qk_norm not in (None, "projection", "head", "head_gain"):
+            raise ValueError(f"normed_gqa_attention: qk_norm must be 'projection', 'head', 'head_gain' or None, got {qk_norm!r}")
         if value_mix not in (None, "source", "blend"):
             raise ValueError(f"normed_gqa_attention: value_mix must be 'source', 'blend' or None, got {value_mix!r}")
         if gate not in ops.HEAD_GATES:
@@ -169,6 +170,9 @@ class NormedGQAAttention(PagedGQAAttention):
         if self.qk_norm == "projection":
             t["q_norm.weight"] = TensorSpec((H * D,), "vector32")
             t["k_norm.weight"] = TensorSpec((G * D,), "vector32")
+        elif self.qk_norm == "head_gain":
+            t["q_norm.weight"] = TensorSpec((D,), "vector32")
+            t["k_norm.weight"] = TensorSpec((D,), "vector32")
         if self.value_mix is not None:
             # (the layer whose values are the source has the scalar too, and does not use it)
             t["value_mix.weight"] = TensorSpec((), "vector32", init=lambda g, shape, device: torch.rand(shape, generator=g, device=device))
@@ -184,7 +188,7 @@ class NormedGQAAttention(PagedGQAAttention):
         self.w_in = rt.prepare_weight(torch.cat(joined, dim=0).contiguous())
         self.cols = (0, H * D, H * D + G * D)
         self.gate_col = H * D + G * D + G * Dv
-        self.q_gain, self.k_gain = weights.get("q_norm.weight"), weights.get("k_norm.weight")
+        self._bind_gains(weights)
         self.mix = weights["value_mix.weight"].reshape(1) if self.value_mix == "blend" else None
         self.w_o = rt.prepare_weight(weights["o.weight"])
         self.position.bind({}, rt)
@@ -192,6 +196,14 @@ class NormedGQAAttention(PagedGQAAttention):
         self.interleaved = getattr(self.position, "layout", "half") == "interleaved"
         if self.rotated_dims and not hasattr(self.position, "rotary_table"):
             raise ValueError("normed_gqa_attention: the position encoding offers no table of cosines and sines")
+
+    def _bind_gains(self, weights):
+        """The gains of the norm over the projection (one per value) or of the heads' own norm (one per head dim)."""
+        per_dim = self.qk_norm == "head_gain"
+        self.q_gain = None if per_dim else weights.get("q_norm.weight")
+        self.k_gain = None if per_dim else weights.get("k_norm.weight")
+        self.q_head_gain = weights.get("q_norm.weight") if per_dim else None
+        self.k_head_gain = weights.get("k_norm.weight") if per_dim else None
 
     def forward(self, x, step, cache):
         rt, n = self.rt, x.shape[0]
@@ -211,9 +223,10 @@ class NormedGQAAttention(PagedGQAAttention):
             mode = 2
         q = rt.buffer("nattn_q", n, H * P)
         ops.qkv_prepare(proj, self.cols, step.positions, step.tok_seq, table, q, cache.kv, H, D, Dv, self.rotated_dims,
-                        self.interleaved, angles, self.q_gain, self.k_gain, self.qk_norm == "head", self.eps,
+                        self.interleaved, angles, self.q_gain, self.k_gain, self.qk_norm in ("head", "head_gain"), self.eps,
                         v_first=v_first, value_mix=mode, mix=self.mix, write_cache=cache.writes,
-                        row_scales=rt.buffer("nattn_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None)
+                        row_scales=rt.buffer("nattn_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None,
+                        q_head_gain=self.q_head_gain, k_head_gain=self.k_head_gain)
         out = rt.buffer("nattn_out", n, H * P)
         self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, softcap=self.softcap)
         if self.gate is not None or P != Dv:
@@ -233,7 +246,13 @@ class MixedHeadsAttention(NormedGQAAttention):
     * ``head_mix``: the heads' scores are mixed by a learned matrix, score_h <- sum_g T[h, g] score_g, after scale
       and bias and before the window's mask and the softmax;
     * ``sink``: a learned number per head whose exponential joins the softmax's denominator once; it has no key
-      and no value.
+      and no value;
+    * the mask: ``window`` newest keys (the base class's), with ``keep_first`` the first tokens of a sequence stay
+      visible to every later query beside the window (at their true positions); ``chunk`` > 0 instead of a window: a
+      query sees the earlier keys of its own run of ``chunk`` positions, counted from position 0 of the sequence;
+    * ``bias``: the projections of q, k and v have biases; ``out_bias``: the output projection has one;
+    * ``values="keys"``: there is no value projection, the values are the keys as projected (bias included, before
+      their norm); key and value size are then equal.
 
     ``own_kv=False``: the layer has no key and value projections (nor their norm); its run-order entry reads the
     cache of an earlier entry with equal head counts and sizes.  ``cache_window``: how many of the newest keys the
@@ -246,13 +265,25 @@ class MixedHeadsAttention(NormedGQAAttention):
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int | None = None,
                  window: int = 0, scale: float | None = None, qk_norm: str | None = None, eps: float = 1e-6,
                  slope_exponent: float | None = None, head_mix: bool = False, sink: bool = False, own_kv: bool = True,
-                 cache_window: int | None = None):
+                 cache_window: int | None = None, keep_first: int = 0, chunk: int = 0, bias: bool = False, out_bias: bool = False,
+                 values: str = "projection"):
+        if values not in ("projection", "keys"):
+            raise ValueError(f"mixed_heads_attention: values must be 'projection' or 'keys', got {values!r}")
+        if values == "keys" and value_dim not in (None, head_dim):
+            raise ConfigError(f"mixed_heads_attention: values that are the keys have the keys' size {head_dim}, not {value_dim}")
+        if chunk and window:
+            raise ConfigError("mixed_heads_attention: a window or chunks, not both")
+        if chunk < 0 or keep_first < 0 or (chunk and keep_first):
+            raise ConfigError(f"mixed_heads_attention: chunks of {chunk} positions with {keep_first} kept first tokens")
+        self.keep_first, self.chunk = int(keep_first), int(chunk)
+        self.has_bias, self.has_out_bias, self.values = bool(bias), bool(out_bias), values
         super().__init__(hidden_size, n_heads, n_kv_heads, head_dim, PartSpec("none", {}), value_dim=value_dim, window=window,
                          scale=scale, qk_norm=qk_norm, eps=eps)
         self.slope_exponent = float(slope_exponent) if slope_exponent is not None else None
         self.head_mix, self.sink, self.own_kv = bool(head_mix), bool(sink), bool(own_kv)
         self.cache_window = self.window if cache_window is None else int(cache_window)
-        if self.cache_window and (not self.window or self.window > self.cache_window):
+        self.cache_chunk = self.chunk if cache_window is None else 0         # (a cache that others read keeps what they ask for)
+        if self.cache_window and ((not self.window and not self.chunk) or self.window > self.cache_window or self.chunk > self.cache_window):
             raise ConfigError(f"mixed_heads_attention: a window of {self.window or 'all'} keys over a cache that keeps {self.cache_window}")
         most = ops.attn_mixed_max_heads(self.stored_dim)
         if n_heads > most:
@@ -260,13 +291,13 @@ class MixedHeadsAttention(NormedGQAAttention):
                               f"kernel holds at once ({most})")
 
     def cache_spec(self):
-        return PagedKVSpec(self.n_kv_heads, self.stored_dim, self.cache_window)
+        return PagedKVSpec(self.n_kv_heads, self.stored_dim, self.cache_window, self.keep_first if self.cache_window else 0, self.cache_chunk)
 
     def signature_group(self):
-        return ("mixed_heads_attention", self.window)
+        return ("mixed_heads_attention", self.window or self.chunk)
 
     def step_signature(self, batch):
-        return self.kernels.signature(batch, self.window)
+        return self.kernels.signature(batch, self.window or self.chunk)       # (how far back a row's own run of keys can reach)
 
     @classmethod
     def step_metadata_for(cls, batch, mixers):
@@ -278,6 +309,14 @@ class MixedHeadsAttention(NormedGQAAttention):
         if not self.own_kv:
             for name in ("k.weight", "v.weight", "k_norm.weight"):
                 t.pop(name, None)
+        if self.values == "keys":
+            t.pop("v.weight", None)
+        if self.has_bias:
+            for name in ("q", "k", "v"):
+                if name + ".weight" in t:
+                    t[name + ".bias"] = TensorSpec((t[name + ".weight"].shape[0],), "vector32", init="normal")
+        if self.has_out_bias:
+            t["o.bias"] = TensorSpec((self.hidden_size,), "vector32", init="normal")
         if self.head_mix:
             eye = lambda g, shape, device: torch.eye(shape[0], device=device) + 0.3 * torch.randn(shape, generator=g, device=device)
             t["talk"] = TensorSpec((H, H), "vector32", init=eye)
@@ -289,11 +328,14 @@ class MixedHeadsAttention(NormedGQAAttention):
         self.rt = rt
         self.kernels = rt.kernels("mixed_heads_attention")
         H, G, D, Dv = self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim
-        joined = [weights["q.weight"]] + ([weights["k.weight"], weights["v.weight"]] if self.own_kv else [])
-        self.w_in = rt.prepare_weight(torch.cat(joined, dim=0).contiguous())
-        self.cols = (0, H * D, H * D + G * D) if self.own_kv else (0, -1, -1)
-        self.q_gain, self.k_gain = weights.get("q_norm.weight"), weights.get("k_norm.weight")
+        names = ["q"] + ((["k"] if self.values == "keys" else ["k", "v"]) if self.own_kv else [])
+        self.w_in = rt.prepare_weight(torch.cat([weights[k + ".weight"] for k in names], dim=0).contiguous())
+        self.b_in = torch.cat([weights[k + ".bias"] for k in names]).contiguous() if self.has_bias else None
+        # (values that are the keys are read from the keys' columns of the projection, as it leaves the product and its bias)
+        self.cols = (0, H * D, H * D if self.values == "keys" else H * D + G * D) if self.own_kv else (0, -1, -1)
+        self._bind_gains(weights)
         self.w_o = rt.prepare_weight(weights["o.weight"])
+        self.b_o = weights.get("o.bias")
         self.talk, self.sinks = weights.get("talk"), weights.get("sink")
         self.slopes = None
         if self.slope_exponent is not None:
@@ -308,14 +350,22 @@ class MixedHeadsAttention(NormedGQAAttention):
         table = step.block_tables[cache.group]
         proj = rt.buffer("amix_proj", n, self.w_in.rows, torch.float32)
         rt.gemm(x, self.w_in, proj)
+        if self.b_in is not None:
+            ops.add_rowvec(proj, self.b_in)
         q = rt.buffer("amix_q", n, H * P)
         ops.qkv_prepare(proj, self.cols, step.positions, step.tok_seq, table, q, cache.kv, H, D, Dv, 0, False, None,
-                        self.q_gain, self.k_gain, self.qk_norm == "head", self.eps, write_cache=cache.writes,
-                        row_scales=rt.buffer("amix_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None)
+                        self.q_gain, self.k_gain, self.qk_norm in ("head", "head_gain"), self.eps, write_cache=cache.writes,
+                        row_scales=rt.buffer("amix_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None,
+                        q_head_gain=self.q_head_gain, k_head_gain=self.k_head_gain)
         out = rt.buffer("amix_out", n, H * P)
-        self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, self.slopes, self.talk, self.sinks)
+        self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, self.slopes, self.talk, self.sinks,
+                               keep_first=self.keep_first, chunk=self.chunk)
         if P != Dv:
             packed = rt.buffer("amix_packed", n, H * Dv)
             ops.heads_gate(out, P, None, 0, None, packed, H)
             out = packed
-        return Product(out, self.w_o)
+        if self.b_o is None:
+            return Product(out, self.w_o)
+        delta = rt.buffer("amix_delta", n, self.hidden_size, torch.float32)
+        rt.gemm(out, self.w_o, delta)
+        return ops.add_rowvec(delta, self.b_o)

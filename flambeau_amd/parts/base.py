@@ -78,23 +78,30 @@ class CacheSpec:
 
 @dataclass(frozen=True)
 class PageGroup:
-    """Key of a group of paged caches.  ``window`` = newest rows still needed, 0 = all."""
+    """Key of a group of paged caches.  ``window`` = newest rows still needed, 0 = all; ``keep_first`` = rows at the
+    start of a request that stay needed whatever the window says; ``chunk`` > 0 (instead of a window) = only the rows
+    of the newest run of ``chunk`` positions, counted from 0, are still needed."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    keep_first: int = 0
+    chunk: int = 0
 
 
 @dataclass(frozen=True)
 class PagedKVSpec(CacheSpec):
     """Per-token rows that grow with the request: keys and values in pages.
-    ``window`` = number of newest keys still needed (0: all).  One (page, kv head) holds
-    ``page_size`` rows of ``head_dim`` values back to back, keys row by row and values transposed."""
+    ``window`` = number of newest keys still needed (0: all); ``keep_first`` and ``chunk`` as in ``PageGroup``.
+    One (page, kv head) holds ``page_size`` rows of ``head_dim`` values back to back, keys row by row and values
+    transposed."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    keep_first: int = 0
+    chunk: int = 0
 
     def page_group(self):
-        return PageGroup(self.n_kv_heads, self.head_dim, self.window)
+        return PageGroup(self.n_kv_heads, self.head_dim, self.window, self.keep_first, self.chunk)
 
     def allocate_pool(self, n_entries, n_pages, page_size, dtype, device):
         return torch.zeros((n_entries, n_pages, 2, self.n_kv_heads, page_size, self.head_dim), dtype=dtype, device=device)

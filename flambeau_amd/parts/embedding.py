@@ -109,6 +109,19 @@ class PositionalTokenEmbedding(TokenEmbedding):
         return out
 
 
+@HEADS.register("capped_linear_head")
+class CappedOutputHead(OutputHead):
+    """logits = cap * tanh((x W^T) / cap), applied to the 32-bit products; ``softcap=None`` leaves them as they are."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, softcap: float | None = None, tied: bool = False):
+        super().__init__(vocab_size, hidden_size, tied)
+        self.softcap = float(softcap) if softcap else None
+
+    def forward(self, x, max_rows):
+        logits = super().forward(x, max_rows)
+        return ops.softcap_inplace(logits, self.softcap) if self.softcap is not None else logits
+
+
 @HEADS.register("scaled_linear_head")
 class ScaledOutputHead(OutputHead):
     """logits = (x W^T) * scale, the factor applied to the 32-bit products."""

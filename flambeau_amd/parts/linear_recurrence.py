@@ -13,6 +13,9 @@ per (token, head) a decay g = exp(-exp(A_log) softplus(W_a h + dt_bias)) and a w
 beta = sigmoid(W_b h); u = beta (v - S^T k) with the decayed S: the memory is corrected towards v at
 the key, not just added to.  Query/key head of head h: h // (heads / qk_heads).  Every head's o is
 divided by its root mean square, times a gain shared by the heads, times silu of a projection.
+Options: a decay per head AND key dim (``decay="key_dim"``: A_log per head, W_a and dt_bias heads x dim wide,
+S <- diag(g) S), the decay's and the output gate's projections as products of two matrices of low rank
+(``decay_rank``, ``gate_rank``), and a sigmoid in place of the silu (``gate``).
 
 HGRN2: the forget gate is a vector per head (one value per key dim) and also decides what is written:
 S <- diag(f) S + (1 - f) v^T, o = S^T q, with f = l + (1 - l) sigmoid(W_f h + b_f) above a learned lower bound
@@ -103,7 +106,17 @@ class GatedDelta(Mixer):
     lazy_input = True
 
     def __init__(self, hidden_size: int, n_heads: int, n_qk_heads: int, head_dim: int, value_dim: int, conv_taps: int, eps: float,
-                 unit_eps: float = 1e-6, query_scale: float | None = None):
+                 unit_eps: float = 1e-6, query_scale: float | None = None, decay: str = "head", decay_rank: int | None = None,
+                 gate_rank: int | None = None, gate: str = "silu"):
+        if decay not in ("head", "key_dim"):
+            raise ValueError(f"gated_delta: decay must be 'head' or 'key_dim', got {decay!r}")
+        if gate not in ("silu", "sigmoid"):
+            raise ValueError(f"gated_delta: gate must be 'silu' or 'sigmoid', got {gate!r}")
+        if decay_rank is not None and decay != "key_dim":
+            raise ConfigError("gated_delta: a decay projection of low rank comes with a decay per key dim")
+        if any(r is not None and r < 1 for r in (decay_rank, gate_rank)):
+            raise ConfigError(f"gated_delta: ranks {decay_rank} and {gate_rank} of the decay's and the gate's projections")
+        self.decay, self.decay_rank, self.gate_rank, self.gate = decay, decay_rank, gate_rank, gate
         if head_dim > ops.linear_scan_max_dim():
             raise ConfigError(f"gated_delta: 'dim' {head_dim} is beyond what the kernel takes ({ops.linear_scan_max_dim()})")
         if not 1 <= conv_taps <= ops.conv_max_taps():
@@ -131,22 +144,34 @@ class GatedDelta(Mixer):
     def tensors(self):
         W, H, G, D, Dv, K = self.hidden_size, self.n_heads, self.n_qk_heads, self.head_dim, self.value_dim, self.conv_taps
         uniform = lambda lo, hi: (lambda g, shape, device: lo + (hi - lo) * torch.rand(shape, generator=g, device=device))
-        return {"q.weight": TensorSpec((G * D, W)), "k.weight": TensorSpec((G * D, W)), "v.weight": TensorSpec((H * Dv, W)),
-                "q_conv.weight": TensorSpec((G * D, K), "vector32", init=uniform(-0.5, 0.5)),
-                "k_conv.weight": TensorSpec((G * D, K), "vector32", init=uniform(-0.5, 0.5)),
-                "v_conv.weight": TensorSpec((H * Dv, K), "vector32", init=uniform(-0.5, 0.5)),
-                "b.weight": TensorSpec((H, W)), "a.weight": TensorSpec((H, W)),
-                "A_log": TensorSpec((H,), "vector32", init=uniform(-3.0, 0.5)),
-                "dt_bias": TensorSpec((H,), "vector32", init=uniform(-2.0, 1.0)),
-                "norm.weight": TensorSpec((Dv,), "vector32"),
-                "g.weight": TensorSpec((H * Dv, W)), "o.weight": TensorSpec((W, H * Dv))}
+        A = H * D if self.decay == "key_dim" else H          # decays per token
+        t = {"q.weight": TensorSpec((G * D, W)), "k.weight": TensorSpec((G * D, W)), "v.weight": TensorSpec((H * Dv, W)),
+             "q_conv.weight": TensorSpec((G * D, K), "vector32", init=uniform(-0.5, 0.5)),
+             "k_conv.weight": TensorSpec((G * D, K), "vector32", init=uniform(-0.5, 0.5)),
+             "v_conv.weight": TensorSpec((H * Dv, K), "vector32", init=uniform(-0.5, 0.5)),
+             "b.weight": TensorSpec((H, W)),
+             "A_log": TensorSpec((H,), "vector32", init=uniform(-3.0, 0.5)),
+             "dt_bias": TensorSpec((A,), "vector32", init=uniform(-2.0, 1.0)),
+             "norm.weight": TensorSpec((Dv,), "vector32"), "o.weight": TensorSpec((W, H * Dv))}
+        if self.decay_rank is not None:
+            t.update({"a1.weight": TensorSpec((self.decay_rank, W)), "a2.weight": TensorSpec((A, self.decay_rank))})
+        else:
+            t["a.weight"] = TensorSpec((A, W))
+        if self.gate_rank is not None:
+            t.update({"g1.weight": TensorSpec((self.gate_rank, W)), "g2.weight": TensorSpec((H * Dv, self.gate_rank))})
+        else:
+            t["g.weight"] = TensorSpec((H * Dv, W))
+        return t
 
     def bind(self, weights, rt):
         self.rt = rt
         H, G, D, Dv = self.n_heads, self.n_qk_heads, self.head_dim, self.value_dim
-        self.w_in = rt.prepare_weight(torch.cat([weights[k + ".weight"] for k in ("q", "k", "v", "b", "a", "g")], dim=0).contiguous())
+        a_name, g_name = ("a1" if self.decay_rank is not None else "a"), ("g1" if self.gate_rank is not None else "g")
+        self.w_in = rt.prepare_weight(torch.cat([weights[k + ".weight"] for k in ("q", "k", "v", "b", a_name, g_name)], dim=0).contiguous())
         self.col_b = self.channels
-        self.col_a, self.col_g = self.col_b + H, self.col_b + 2 * H
+        self.col_a = self.col_b + H
+        self.col_g = self.col_a + weights[a_name + ".weight"].shape[0]
+        self.w_a2, self.w_g2 = weights.get("a2.weight"), weights.get("g2.weight")     # (second factors: read row by row as they are stored)
         self.conv_w = torch.cat([weights[k + "_conv.weight"] for k in ("q", "k", "v")], dim=0).contiguous()
         self.a_log, self.dt_bias = weights["A_log"], weights["dt_bias"]
         self.norm = weights["norm.weight"].repeat(H).contiguous()          # one gain for every head, laid out heads x vdim
@@ -159,14 +184,26 @@ class GatedDelta(Mixer):
         rt.gemm(x, self.w_in, proj)
         prep = rt.buffer("gd_prep", n, self.channels, torch.float32)
         gates = rt.buffer("gd_gates", n, 2 * H, torch.float32)
-        ops.conv_prepare(proj, 0, self.col_b, self.col_a, self.conv_w, self.a_log, self.dt_bias, cache.state, self.conv_at,
-                         step.tok_seq, step.seq_q_start, step.seq_q_len, step.seq_slots, prep, gates, G, H, D, Dv,
+        per_dim = self.decay == "key_dim"
+        ops.conv_prepare(proj, 0, self.col_b, self.col_a, self.conv_w, None if per_dim else self.a_log, self.dt_bias, cache.state,
+                         self.conv_at, step.tok_seq, step.seq_q_start, step.seq_q_len, step.seq_slots, prep, gates, G, H, D, Dv,
                          self.conv_taps, self.query_scale, self.unit_eps)
+        key_decay = None
+        if per_dim:
+            # the decays per head and key dim: exp(-exp(A_log) softplus(a + dt_bias)), a straight from the joined
+            # projection or through the second factor of a projection of low rank (its first factor's products in 32-bit)
+            a, col = proj, self.col_a
+            if self.w_a2 is not None:
+                a, col = ops.lowrank_expand(proj, self.col_a, self.w_a2, rt.buffer("gd_decay_in", n, H * D, torch.float32)), 0
+            key_decay = ops.channel_decay(a, col, self.a_log, self.dt_bias, rt.buffer("gd_decay", n, H * D, torch.float32), H, D)
         hidden = rt.buffer("gd_hidden", n, H * Dv, torch.float32)
         ops.linear_scan(prep[:, :G * D], prep[:, G * D:2 * G * D], prep[:, 2 * G * D:], cache.state, step.seq_q_start,
-                        step.seq_q_len, step.seq_slots, hidden, H, G, D, Dv, token_gates=gates)
+                        step.seq_q_len, step.seq_slots, hidden, H, G, D, Dv, token_gates=gates, key_decay=key_decay)
+        gate_rows, gate_col = proj, self.col_g
+        if self.w_g2 is not None:
+            gate_rows, gate_col = ops.lowrank_expand(proj, self.col_g, self.w_g2, rt.buffer("gd_gate_in", n, H * Dv, torch.float32)), 0
         out = rt.buffer("gd_out", n, H * Dv)
-        ops.headnorm_gate(hidden, self.norm, proj, self.col_g, out, H, self.eps, gate_kind="silu")
+        ops.headnorm_gate(hidden, self.norm, gate_rows, gate_col, out, H, self.eps, gate_kind=self.gate)
         return Product(out, self.w_o)
 
 

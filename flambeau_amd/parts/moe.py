@@ -64,10 +64,28 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden_size: int, n_experts: int, top: int, expert_size: int, shared_size: int | None = None,
                  scoring: str = "sigmoid", renormalise: bool = False, weight_on: str = "input", shared_gate: bool = True,
-                 gated: bool = True, activation: str = "silu", router_bias: bool = False):
-        """``scoring``: ``sigmoid``, ``softmax`` (over all experts) or ``softmax_chosen`` (over the chosen logits only);
-        ``gated=False``: an expert is W_down act(W_up u) with ``activation`` (no gate matrix); ``router_bias``: the
-        router's logits have a bias."""
+                 gated: bool = True, activation: str = "silu", router_bias: bool = False, correction: bool = False,
+                 n_groups: int = 1, keep_groups: int = 1, n_identity: int = 0, weight_scale: float = 1.0):
+        """``scoring``: ``sigmoid``, ``softmax`` (over all experts), ``softmax_chosen`` (over the chosen logits only) or
+        ``softmax_grouped``; ``gated=False``: an expert is W_down act(W_up u) with ``activation`` (no gate matrix);
+        ``router_bias``: the router's logits have a bias.
+
+        ``softmax_grouped``: scores s = softmax over ALL the router's outputs; the choice goes by s + a learned
+        ``correction`` per output (if ``correction``), the weights by s alone; the outputs form ``n_groups`` equal groups of
+        neighbours, a group's score is its largest choice score, and only outputs of the ``keep_groups`` best groups can
+        be chosen; the weights are the chosen scores over their sum (+ 1e-20) times ``weight_scale``.  The last
+        ``n_identity`` outputs of the router are identity experts: they have no matrices and return their input (times
+        the weight); the router then has ``n_experts + n_identity`` outputs, and groups are formed over all of them."""
+        grouped = scoring == "softmax_grouped"
+        if not grouped and (correction or n_groups != 1 or keep_groups != 1 or n_identity or weight_scale != 1.0):
+            raise ValueError("routed_experts: correction, groups, identity experts and a weight scale come with scoring 'softmax_grouped'")
+        n_outputs = n_experts + int(n_identity)
+        if grouped and (n_groups < 1 or n_outputs % n_groups or not 1 <= keep_groups <= n_groups or keep_groups * (n_outputs // n_groups) < top):
+            raise ValueError(f"routed_experts: {keep_groups} of {n_groups} groups over {n_outputs} router outputs cannot give {top} choices")
+        if grouped and (weight_on != "output" or router_bias):
+            raise ValueError("routed_experts: scoring 'softmax_grouped' weights the experts' outputs and has no router bias")
+        self.grouped, self.correction, self.n_groups, self.keep_groups = grouped, bool(correction), int(n_groups), int(keep_groups)
+        self.n_identity, self.n_outputs, self.weight_scale = int(n_identity), n_outputs, float(weight_scale)
         if weight_on not in ("input", "output"):
             raise ValueError(f"routed_experts: weight_on must be 'input' or 'output', got {weight_on!r}")
         if scoring not in ops.ROUTER_SCORINGS:
@@ -84,7 +102,9 @@ class RoutedExperts(FeedForward):
 
     def tensors(self):
         W, F = self.hidden_size, self.expert_size
-        t = {"router.weight": TensorSpec((self.n_experts, W))}
+        t = {"router.weight": TensorSpec((self.n_outputs, W))}
+        if self.correction:
+            t["correction"] = TensorSpec((self.n_outputs,), "vector32", init="normal")
         if self.router_bias:
             t["router.bias"] = TensorSpec((self.n_experts,), "vector32", init="normal")
         for e in range(self.n_experts):
@@ -113,6 +133,7 @@ class RoutedExperts(FeedForward):
             extra = self.w_logits.shape[0] - E
             self.b_logits = torch.cat([weights["router.bias"], torch.zeros(extra, dtype=torch.float32, device=weights["router.bias"].device)]).contiguous()
         self.w_down = torch.stack([weights[f"e{e}.down.weight"] for e in range(E)]).contiguous()
+        self.correction_w = weights.get("correction")
         if self.shared_size is not None:
             self.ws_gate_up = rt.prepare_gate_up(weights["shared.gate.weight"], weights["shared.up.weight"])
             self.ws_down = rt.prepare_weight(weights["shared.down.weight"])
@@ -131,9 +152,13 @@ class RoutedExperts(FeedForward):
         src_row = ints("moe_src_row", pairs, 1, most).view(-1)
         src_scale = rt.buffer("moe_src_scale", pairs, 1, torch.float32, max_rows=most).view(-1)
         pair_w = rt.buffer("moe_pair_w", pairs, 1, torch.float32, max_rows=most).view(-1)
-        n_tiles = ops.moe_max_tiles(pairs, E)
-        tiles = ints("moe_tiles", n_tiles, 4, ops.moe_max_tiles(most, E))
-        ops.moe_route(logits, 0, E, top, place, src_row, src_scale, pair_w, tiles, self.scoring, self.renormalise)
+        n_tiles = ops.moe_max_tiles(pairs, self.n_outputs)
+        tiles = ints("moe_tiles", n_tiles, 4, ops.moe_max_tiles(most, self.n_outputs))
+        if self.grouped:
+            ops.moe_route_grouped(logits, 0, self.n_outputs, self.n_identity, top, self.correction_w, self.n_groups, self.keep_groups,
+                                  self.weight_scale, place, src_row, src_scale, pair_w, tiles)
+        else:
+            ops.moe_route(logits, 0, E, top, place, src_row, src_scale, pair_w, tiles, self.scoring, self.renormalise)
         on_input = self.weight_on == "input"
         gate_up = rt.buffer("moe_gate_up", pairs, (2 if self.gated else 1) * F, torch.float32, max_rows=most)
         ops.moe_gemm(x, self.w_gate_up, gate_up, tiles, src_row, src_scale if on_input else None, matrix_cores=rt.tuned)
@@ -144,6 +169,8 @@ class RoutedExperts(FeedForward):
             ops.activation(gate_up, act, self.activation)
         y = rt.buffer("moe_y", pairs, W, torch.float32, max_rows=most)
         ops.moe_gemm(act, self.w_down, y, tiles, None, None if on_input else src_scale, matrix_cores=rt.tuned)
+        if self.n_identity:
+            ops.moe_identity(x, src_row, src_scale, y, tiles)          # (the rows of identity experts: weight * input)
         shared = None
         if self.shared_size is not None:
             sact = rt.buffer("moe_shared_act", n, self.shared_size)
@@ -151,5 +178,5 @@ class RoutedExperts(FeedForward):
             shared = rt.buffer("moe_shared", n, W, torch.float32)
             rt.gemm(sact, self.ws_down, shared)
         delta = rt.buffer("moe_delta", n, W, torch.float32)
-        ops.moe_combine(y, place, top, delta, shared=shared, gate=logits if self.shared_gate else None, gate_col=E)
+        ops.moe_combine(y, place, top, delta, shared=shared, gate=logits if self.shared_gate else None, gate_col=self.n_outputs)
         return delta

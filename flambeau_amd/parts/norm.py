@@ -11,16 +11,19 @@ from .base import NORMS, Norm, TensorSpec
 class RMSNorm(Norm):
     replayable = True
 
-    def __init__(self, hidden_size: int, eps: float):
+    def __init__(self, hidden_size: int, eps: float, unit_offset: bool = False):
+        """``unit_offset``: the weight is stored around zero and the gain is one plus it, y = x / rms(x) * (1 + w)."""
         self.hidden_size = hidden_size
         self.eps = eps
+        self.unit_offset = bool(unit_offset)
 
     def tensors(self):
-        return {"weight": TensorSpec((self.hidden_size,), "vector32")}
+        return {"weight": TensorSpec((self.hidden_size,), "vector32", init="normal" if self.unit_offset else None)}
 
     def bind(self, weights, rt):
         self.rt = rt
-        self.weight = weights["weight"]
+        # (``weight`` is the gain as it multiplies: every kernel that norms, fused or not, reads this one vector)
+        self.weight = (weights["weight"] + 1.0).contiguous() if self.unit_offset else weights["weight"]
 
     def forward(self, x, out, delta=None, store_sum=False, rows=None):
         return ops.rmsnorm(x, self.weight, out, self.eps, delta=delta, store_sum=store_sum, rows=rows)

@@ -1,7 +1,8 @@
 """Two mixers side by side: both read the same normed input, each output is normed over the model width
 (root mean square, eps inside the root, a plain gain of its own) and the results are added with a factor
-each (a half each: their mean).  The members are any registered mixers; one of them may keep pages, the
-others records per slot, which the joined cache lays side by side."""
+each (a half each: their mean); with ``normed=False`` the outputs are added as they are, each with its factor.
+The members are any registered mixers; one of them may keep pages, the others records per slot, which the
+joined cache lays side by side."""
 from __future__ import annotations
 
 import torch
@@ -19,8 +20,8 @@ class SideBySide(Mixer):
     def lazy_input(self):
         return all(m.lazy_input for m in self._members.values())
 
-    def __init__(self, hidden_size: int, left: PartSpec, right: PartSpec, eps: float, factors=(0.5, 0.5)):
-        self.hidden_size, self.eps = hidden_size, float(eps)
+    def __init__(self, hidden_size: int, left: PartSpec, right: PartSpec, eps: float = 0.0, factors=(0.5, 0.5), normed: bool = True):
+        self.hidden_size, self.eps, self.normed = hidden_size, float(eps), bool(normed)
         self.factors = (float(factors[0]), float(factors[1]))
         self.left, self.right = MIXERS.create(left), MIXERS.create(right)
         self._members = {"left": self.left, "right": self.right}
@@ -54,15 +55,16 @@ class SideBySide(Mixer):
 
     def tensors(self):
         t = {f"{p}.{name}": spec for p, m in self._members.items() for name, spec in m.tensors().items()}
-        t["left_out.weight"] = TensorSpec((self.hidden_size,), "vector32")
-        t["right_out.weight"] = TensorSpec((self.hidden_size,), "vector32")
+        if self.normed:
+            t["left_out.weight"] = TensorSpec((self.hidden_size,), "vector32")
+            t["right_out.weight"] = TensorSpec((self.hidden_size,), "vector32")
         return t
 
     def bind(self, weights, rt):
         self.rt = rt
         for p, m in self._members.items():
             m.bind({k[len(p) + 1:]: v for k, v in weights.items() if k.startswith(p + ".")}, rt)
-        self.gain_left, self.gain_right = weights["left_out.weight"], weights["right_out.weight"]
+        self.gain_left, self.gain_right = weights.get("left_out.weight"), weights.get("right_out.weight")
 
     def _member_cache(self, cache: LayerCache, index: int):
         """What a member sees: the pages as they are, and its own stretch of the slot's record."""
@@ -87,5 +89,8 @@ class SideBySide(Mixer):
                 d = d.compute(rt, out=rt.buffer("sbs_" + name, n, W, torch.float32))
             outs.append(d)
         delta = rt.buffer("sbs_delta", n, W, torch.float32)
-        ops.norm_mix(outs[0], self.gain_left, self.factors[0], outs[1], self.gain_right, self.factors[1], delta, self.eps)
+        if self.normed:
+            ops.norm_mix(outs[0], self.gain_left, self.factors[0], outs[1], self.gain_right, self.factors[1], delta, self.eps)
+        else:
+            ops.scaled_sum(outs[0], self.factors[0], outs[1], self.factors[1], delta)
         return delta

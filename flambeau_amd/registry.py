@@ -50,8 +50,25 @@ def config_from_dict(raw: dict, where: str = "config.json"):
 
 
 def config_from_dir(model_dir):
+    """``(Architecture, typed config)`` of a model folder.  A configuration class with ``sizes_from_tensors(raw, shapes)``
+    is given the shapes of the folder's tensors first (read from the files' headers), for sizes that no key of
+    config.json holds."""
     raw = read_config_json(model_dir)
-    return config_from_dict(raw, f"{model_dir}/config.json")
+    where = f"{model_dir}/config.json"
+    arch = find_architecture(architecture_name(raw, where))
+    fill = getattr(arch.config_class, "sizes_from_tensors", None)
+    if fill is not None:
+        from .weights.loader import SafetensorsDir, WeightFileError
+        try:
+            src = SafetensorsDir(model_dir)
+        except WeightFileError:
+            src = None                  # (a folder without weights: the configuration must then say everything itself)
+        if src is not None:
+            try:
+                raw = fill(raw, {name: tuple(src.info(name)[0]) for name in src.names()})
+            finally:
+                src.close()
+    return arch, arch.config_class.from_dict(raw, where)
 
 
 def _load_builtin():
