@@ -66,8 +66,7 @@ class DecoderModel:
         self.final_norm = NORMS.create(spec.final_norm)
         self.head = HEADS.create(spec.head or PartSpec("linear_head", dict(sizes, tied=spec.tied_head)))
         self._signature_mixers = None
-        self._stream_ones = (torch.ones(spec.residual_streams, dtype=torch.float32, device=rt.device)
-                             if spec.residual_streams is not None else None)
+        self._stream_ones = None            # a one per copy of the residual stream, on the device (made when the tensors are bound)
         self._recorded_blocks = None        # per block: can its launches be recorded?
         seen: dict = {}
         self._visits = []                   # per run-order entry: how many earlier entries ran the same layer
@@ -111,6 +110,8 @@ class DecoderModel:
             block.bind(per_owner.get(li, {}), self.rt)
         self.final_norm.bind(per_owner.get("final_norm", {}), self.rt)
         self.head.bind(per_owner.get("head", {}), self.rt, embedding_table=self.embedding.weight)
+        if self.spec.residual_streams is not None:
+            self._stream_ones = torch.ones(self.spec.residual_streams, dtype=torch.float32, device=self.rt.device)
 
     # ------------------------------------------------------------ cache needs
     def cache_entries(self):

@@ -226,7 +226,7 @@ def forward(config, t, tokens, layer_outputs=None):
     t = {k: np.asarray(v, dtype=np.float64) for k, v in t.items()}
     eps = config["norm"]["eps"]
     S = config.get("streams")                       # absent: one stream and the plain residual sum
-    x = embed(tokens, t, config["embedding"]["scale"])
+    x = embed(tokens, t, (config.get("embedding") or {}).get("scale", 1.0))
     xs = np.repeat(x[None], S, axis=0) if S is not None else None
     for l, layer in enumerate(config["layers"]):
         p, m = f"l{l}.", layer["mixer"]
