@@ -29,6 +29,11 @@ beside a Mistral of the same width, head count and number of layers, measured th
 ``--config fitevik``: the Fitevik design (layer norms behind the sublayers, learned positions, the HGRN2 recurrence,
 attention inside a window with a distance bias, mixed heads and a sink, one layer reading another's keys, dense and
 routed feed-forwards with the squared relu) at two sizes, six layers, beside the same Mistral; a line of the same shape.
+
+``--config lenedra``: the Lenedra design (a residual stream in four copies, attention whose keys are its values inside a
+window that keeps the first tokens, chunked attention with a sink beside a delta rule with decays per key dim, a grouped
+router with identity experts and a shared expert) at two sizes, six layers, beside the closest design the engine has,
+Fitevik, at the same widths, head counts, windows and experts; a line of the same shape.
 """
 from __future__ import annotations
 
@@ -417,6 +422,28 @@ FITEVIK_SIZES = {
 }
 
 
+def lenedra_config(width, heads, kv_heads, ff, experts, top, expert_ff, rec_heads, window, vocab=32768):
+    att = {"type": "attention", "mixer": dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5,
+                                              mask={"size": window, "keep_first": 4})}
+    left = dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, mask={"size": window})
+    right = dict(heads=rec_heads, kv_heads=rec_heads // 2, dim=128, vdim=128, conv=4, decay_rank=64, gate_rank=64)
+    par = {"type": "parallel", "mixer": dict(left=left, right=right, left_scale=0.5, right_scale=1.0)}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": experts, "identity": 2, "top": top, "groups": {"count": 2, "keep": 1}, "scale": 2.5},
+           "expert": {"ff": expert_ff}, "shared": {"ff": expert_ff}}
+    layers = [dict(att, mlp=dense), dict(par, mlp=moe), dict(att, mlp=dense), dict(par, mlp=moe), dict(att, mlp=moe), dict(par, mlp=dense)]
+    return {"architecture": "Lenedra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": width ** 0.5},
+            "logit_softcap": 30.0, "streams": 4, "layers": layers}
+
+
+def bench_lenedra(a, dtype_name):
+    """The same for the Lenedra design: three attention layers and three pairs (chunked attention beside the delta rule),
+    three dense and three routed feed-forwards, beside Fitevik (three recurrent and three attention layers, three dense
+    and three routed feed-forwards) at the same sizes."""
+    return bench_design(a, dtype_name, "lenedra", "Lenedra", FITEVIK_SIZES, lenedra_config, "6 layers",
+                        beside=lambda sz: ("fitevik", fitevik_config(**sz)), beside_title="Fitevik")
+
+
 def bench_fitevik(a, dtype_name):
     """The same for the Fitevik design: three recurrent and three attention layers (one reads another's keys)."""
     return bench_design(a, dtype_name, "fitevik", "Fitevik", FITEVIK_SIZES, fitevik_config, "6 layers")
@@ -433,7 +460,9 @@ def bench_bugidra(a, dtype_name):
     return bench_design(a, dtype_name, "bugidra", "Bugidra", BUGIDRA_SIZES, bugidra_config, "6 layers")
 
 
-def bench_design(a, dtype_name, design, title, all_sizes, make_config, runs_text):
+def bench_design(a, dtype_name, design, title, all_sizes, make_config, runs_text, beside=None, beside_title="Mistral"):
+    """``beside(sizes) -> (label, configuration)``: the model the design is measured beside (a Mistral of equal width, head
+    count and number of layers if none is given)."""
     import torch
     from flambeau_amd import random_model
     points = {}
@@ -444,7 +473,7 @@ def bench_design(a, dtype_name, design, title, all_sizes, make_config, runs_text
         runs = 6           # layer runs of either design's configuration
         mcfg = dict(_BASE, num_hidden_layers=runs, hidden_size=sz["width"], num_attention_heads=sz["heads"], num_key_value_heads=8,
                     head_dim=128, intermediate_size=sz["ff"], vocab_size=32768, rope_theta=1e6, sliding_window=None)
-        for label, cfg in ((design, kcfg), ("mistral", mcfg)):
+        for label, cfg in ((design, kcfg), beside(sz) if beside is not None else ("mistral", mcfg)):
             if a.only_model and a.only_model != label:
                 continue
             model, _ = random_model(cfg, seed=0, dtype=dtype_name, max_batch_tokens=PROMPT_LEN + 64, std=0.02, gain_std=0.0)
@@ -465,7 +494,7 @@ def bench_design(a, dtype_name, design, title, all_sizes, make_config, runs_text
            "value": head, "unit": "tokens/s", "n_gpus": 1, "steps": 24, "warmup": 6,
            "ms_per_step": points.get(f"w4096_{design}_decode_b8_ms"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": a.dtype, "data": "synthetic: random weights N(0, 0.02^2), uniform random token ids, caches filled with random values for decode",
-           "config": {"model": f"{title} design at two sizes beside Mistral of equal width", "sizes": all_sizes,
+           "config": {"model": f"{title} design at two sizes beside {beside_title} of equal width", "sizes": all_sizes,
                       "global_batch": 8, "seq_len": PROMPT_LEN, "parallelism": "single GPU"},
            "points": points}
     print(json.dumps(out), flush=True)
@@ -479,10 +508,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--reps", type=int, default=REPS, help="repetitions of the timed steps; the median is reported")
-    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra", "bugidra", "fitevik"])
-    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra / bugidra / fitevik: one size only")
-    ap.add_argument("--only-model", default=None, choices=["kuvidra", "bugidra", "fitevik", "mistral"],
-                    help="--config kuvidra / bugidra / fitevik: one of the two models only")
+    ap.add_argument("--config", default="7b", choices=sorted(CONFIGS) + ["kuvidra", "bugidra", "fitevik", "lenedra"])
+    ap.add_argument("--only-size", default=None, choices=sorted(KUVIDRA_SIZES), help="--config kuvidra / bugidra / fitevik / lenedra: one size only")
+    ap.add_argument("--only-model", default=None, choices=["kuvidra", "bugidra", "fitevik", "lenedra", "mistral"],
+                    help="--config kuvidra / bugidra / fitevik / lenedra: one of the two models only")
     ap.add_argument("--layers", type=int, default=None, help="run only the first layers (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -503,6 +532,8 @@ def main():
         return bench_bugidra(a, dtype_name)
     if a.config == "fitevik":
         return bench_fitevik(a, dtype_name)
+    if a.config == "lenedra":
+        return bench_lenedra(a, dtype_name)
     label, cfg = CONFIGS[a.config]
     if a.config != "7b":
         return bench_serving(a, a.config, label, cfg, dtype_name, el)

@@ -453,7 +453,7 @@ def test_the_stream_after_every_layer(dirs, name, dtype):
         if dtype == "float32":
             assert err.max() < 2e-5, f"layer {i}"
         else:               # (a token whose choice of experts is a close call may turn the other way in bfloat16, and is then far off)
-            assert np.median(err) < 3e-2 and (err > 1e-1).mean() <= 0.2, f"layer {i}"
+            assert np.median(err) < 5e-2 and (err > 1e-1).mean() <= 0.2, f"layer {i}"
 
 
 # ---------------------------------------------------------------- whole models in every cutting
