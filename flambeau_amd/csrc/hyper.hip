@@ -28,16 +28,22 @@ struct HyperStep {
     const int* rows;                // picks the tokens that are read (one output row each), or null; only without y
 };
 
-template <typename T>
-__global__ __launch_bounds__(256) void hyper_step_kernel(HyperStep a, T* __restrict__ normed) {
+// A block per token.  NT threads, each VEC neighbouring values of a row at a time (one 16-byte access where the width
+// allows it); all copies of those values are asked for before the first is used.  The first KEEP turns of the walk over
+// a row keep their u in registers for the norm (a row up to NT * VEC * KEEP wide is read once); what lies beyond is read
+// back from u_out.  SMAX bounds the copies at compile time (4 or 16).  Rows of two thousand values or more take blocks of
+// 1,024 threads, so that a row is a turn or two and a step of few rows is as long as one trip to memory and back.  The
+// block's shape follows from the width alone, never from the step's rows: a row's bits do not depend on its neighbours.
+template <typename T, int NT, int VEC, int KEEP, int SMAX>
+__global__ __launch_bounds__(NT) void hyper_step_kernel(HyperStep a, T* __restrict__ normed) {
     __shared__ float coef[HY_MAX_STREAMS * HY_MAX_STREAMS + 2 * HY_MAX_STREAMS];
-    __shared__ float lds[4];
+    __shared__ float lds[NT / 64];
     const int S = a.S, W = a.W;
     float* mixs = coef;                               // [from][to]
     float* outs = coef + HY_MAX_STREAMS * HY_MAX_STREAMS;
     float* ins = outs + HY_MAX_STREAMS;
-    for (int e = threadIdx.x; e < S * S; e += 256) mixs[e] = a.y ? a.mix[e] : 0.f;
-    for (int e = threadIdx.x; e < S; e += 256) {
+    for (int e = threadIdx.x; e < S * S; e += NT) mixs[e] = a.y ? a.mix[e] : 0.f;
+    for (int e = threadIdx.x; e < S; e += NT) {
         outs[e] = a.y ? a.out_w[e] : 0.f;
         ins[e] = a.in_w ? a.in_w[e] : 0.f;
     }
@@ -47,41 +53,67 @@ __global__ __launch_bounds__(256) void hyper_step_kernel(HyperStep a, T* __restr
     float* x = a.xs + (size_t)t * S * W;
     const float* yr = a.y ? a.y + (size_t)t * W : nullptr;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < W; i += 256) {
-        float old[HY_MAX_STREAMS], now[HY_MAX_STREAMS];
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    // the values c .. c + VEC - 1 of every copy: write the new copies, return u
+    auto turn = [&](int c) {
+        vec_t old[SMAX];
 #pragma unroll
-        for (int s = 0; s < HY_MAX_STREAMS; ++s) old[s] = s < S ? x[(size_t)s * W + i] : 0.f;
-        float u = 0.f;
+        for (int s = 0; s < SMAX; ++s)
+            if (s < S) old[s] = *(const vec_t*)(x + (size_t)s * W + c);
+        vec_t u = 0.f;
         if (yr) {
-            const float yv = yr[i];
+            const vec_t yv = *(const vec_t*)(yr + c);
 #pragma unroll
-            for (int to = 0; to < HY_MAX_STREAMS; ++to) {
+            for (int to = 0; to < SMAX; ++to) {
                 if (to >= S) break;
-                float v = 0.f;
+                vec_t v = 0.f;
 #pragma unroll
-                for (int s = 0; s < HY_MAX_STREAMS; ++s)
-                    if (s < S) v = fmaf(mixs[s * S + to], old[s], v);
-                now[to] = fmaf(outs[to], yv, v);
-                x[(size_t)to * W + i] = now[to];
+                for (int s = 0; s < SMAX; ++s)
+                    if (s < S) v += mixs[s * S + to] * old[s];
+                v += outs[to] * yv;
+                *(vec_t*)(x + (size_t)to * W + c) = v;
+                u += ins[to] * v;
             }
         } else {
 #pragma unroll
-            for (int s = 0; s < HY_MAX_STREAMS; ++s) now[s] = old[s];
+            for (int s = 0; s < SMAX; ++s)
+                if (s < S) u += ins[s] * old[s];
         }
-        if (a.in_w) {
+        return u;
+    };
+    vec_t kept[KEEP];
 #pragma unroll
-            for (int s = 0; s < HY_MAX_STREAMS; ++s)
-                if (s < S) u = fmaf(ins[s], now[s], u);
-            if (a.u_out) a.u_out[(size_t)r * W + i] = u;
-            ss = fmaf(u, u, ss);
-        }
+    for (int k = 0; k < KEEP; ++k) {
+        const int c = (k * NT + threadIdx.x) * VEC;
+        kept[k] = 0.f;
+        if (c >= W) continue;
+        kept[k] = turn(c);
+        if (a.in_w && a.u_out) *(vec_t*)(a.u_out + (size_t)r * W + c) = kept[k];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) ss = fmaf(kept[k][i], kept[k][i], ss);
+    }
+    for (int c = (KEEP * NT + threadIdx.x) * VEC; c < W; c += NT * VEC) {
+        const vec_t u = turn(c);
+        if (a.in_w && a.u_out) *(vec_t*)(a.u_out + (size_t)r * W + c) = u;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) ss = fmaf(u[i], u[i], ss);
     }
     if (!a.in_w || !a.gain) return;
-    ss = block_sum<4>(ss, lds);                       // (the barrier inside also orders this block's u_out stores before its reads)
+    ss = block_sum<NT / 64>(ss, lds);                 // (the barrier inside also orders this block's u_out stores before its reads)
     const float inv = 1.0f / sqrtf(ss / (float)W + a.eps);
-    for (int i = threadIdx.x; i < W; i += 256)
-        normed[(size_t)r * W + i] = from_f32<T>(a.u_out[(size_t)r * W + i] * inv * a.gain[i]);
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int c = (k * NT + threadIdx.x) * VEC;
+        if (c >= W) continue;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) normed[(size_t)r * W + c + i] = from_f32<T>(kept[k][i] * inv * a.gain[c + i]);
+    }
+    for (int c = (KEEP * NT + threadIdx.x) * VEC; c < W; c += NT * VEC)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) normed[(size_t)r * W + c + i] = from_f32<T>(a.u_out[(size_t)r * W + c + i] * inv * a.gain[c + i]);
 }
+
+#define HY_WIDE_ROW 2048      // from this many values a row a block has 1,024 threads
 
 extern "C" int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* mix, const float* out_w,
                              const float* in_w, const int* rows, int n_rows, float* u_out, const float* gain, float eps,
@@ -90,12 +122,25 @@ extern "C" int fl_hyper_step(float* xs, int n, int S, int W, const float* y, con
     FL_CHECK(!y || (mix && out_w), "hyper_step: a sublayer's output without its numbers");
     FL_CHECK(!gain || (in_w && u_out && normed), "hyper_step: a norm needs what it reads and where it writes");
     FL_CHECK(!rows || !y, "hyper_step: picked rows are read only");
+    FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "hyper_step: unknown dtype %d", out_dtype);
     const int blocks = rows ? n_rows : n;
     if (blocks <= 0) return 0;
     HyperStep a{xs, S, W, y, mix, out_w, in_w, u_out, gain, eps, rows};
-    if (out_dtype == FL_F32) hyper_step_kernel<float><<<blocks, 256, 0, stream>>>(a, (float*)normed);
-    else if (out_dtype == FL_BF16) hyper_step_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, (bf16_t*)normed);
-    else FL_CHECK(false, "hyper_step: unknown dtype %d", out_dtype);
+    const bool few = W >= HY_WIDE_ROW, wide = W % 4 == 0, small = S <= 4;
+#define FL_HY(T, NT, VEC, KEEP, SMAX) hyper_step_kernel<T, NT, VEC, KEEP, SMAX><<<blocks, NT, 0, stream>>>(a, (T*)normed)
+#define FL_HY_S(T, NT, VEC, KEEP) do { if (small) FL_HY(T, NT, VEC, KEEP, 4); else FL_HY(T, NT, VEC, KEEP, HY_MAX_STREAMS); } while (0)
+#define FL_HY_T(T)                                   \
+    do {                                             \
+        if (few && wide) FL_HY_S(T, 1024, 4, 2);     \
+        else if (few) FL_HY_S(T, 1024, 1, 4);        \
+        else if (wide) FL_HY_S(T, 256, 4, 4);        \
+        else FL_HY_S(T, 256, 1, 8);                  \
+    } while (0)
+    if (out_dtype == FL_F32) FL_HY_T(float);
+    else FL_HY_T(bf16_t);
+#undef FL_HY_T
+#undef FL_HY_S
+#undef FL_HY
     FL_LAUNCH_CHECK();
     return 0;
 }

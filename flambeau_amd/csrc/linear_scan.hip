@@ -252,8 +252,9 @@ extern "C" int fl_channel_decay(const float* a, int ld, int col, const float* a_
 }
 FL_RECORDABLE(fl_channel_decay)
 
-// out[t][f] = sum_r x[t][col + r] * w[f][r] for a short run of r (the second factor of a projection of low rank):
-// x float rows, w in its storage type, float sums in rising order of r
+// out[t][f] = sum_r x[t][col + r] * wt[r][f] for a short run of r (the second factor of a projection of low rank, given
+// TRANSPOSED, [rank][features], so that neighbouring threads read neighbouring values): x float rows, wt in its
+// storage type, float sums in rising order of r
 template <typename T>
 __global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __restrict__ x, int ld, int col, const T* __restrict__ w,
                                                              float* __restrict__ out, int N, int R) {
@@ -263,9 +264,8 @@ __global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __rest
     __syncthreads();
     const int f = blockIdx.x * 256 + threadIdx.x;
     if (f >= N) return;
-    const T* wr = w + (size_t)f * R;
     float s = 0.f;
-    for (int r = 0; r < R; ++r) s = fmaf(xr[r], to_f32(wr[r]), s);
+    for (int r = 0; r < R; ++r) s = fmaf(xr[r], to_f32(w[(size_t)r * N + f]), s);
     out[(size_t)t * N + f] = s;
 }
 

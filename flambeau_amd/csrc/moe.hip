@@ -88,31 +88,32 @@ __global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__
 // s + correction (correction may be null); the outputs form n_groups equal groups of neighbours, a group's score is
 // its largest choice score, and only outputs of the keep_groups best groups (the lower index among equals) can be
 // chosen; the weights are the chosen s divided by their sum (+ 1e-20) times scale.  A wave per token.
+template <int NU>
 __global__ __launch_bounds__(256) void moe_pick_grouped_kernel(const float* __restrict__ logits, int ld, int col0, int n, int E,
                                                                int top, const float* __restrict__ correction, int n_groups,
                                                                int keep_groups, float scale, int* __restrict__ place,
                                                                float* __restrict__ pair_w) {
     const int lane = threadIdx.x & 63;
-    const int nu = (E + 63) >> 6;
+    constexpr int nu = NU;                         // outputs per lane (lane, lane + 64, ...): E <= 64 * NU
     const int per = E / n_groups;
     for (int t = blockIdx.x * 4 + (threadIdx.x >> 6); t < n; t += gridDim.x * 4) {
         const float* z = logits + (size_t)t * ld + col0;
-        float sv[MOE_MAX_EXPERTS / 64], cv[MOE_MAX_EXPERTS / 64];
+        float sv[NU], cv[NU];
         float zmax = -INFINITY, zsum = 0.f;
 #pragma unroll
-        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+        for (int u = 0; u < NU; ++u) {
             sv[u] = (u < nu && lane + 64 * u < E) ? z[lane + 64 * u] : -INFINITY;
             if (u < nu) zmax = fmaxf(zmax, sv[u]);
         }
         zmax = wave_max(zmax);
 #pragma unroll
-        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+        for (int u = 0; u < NU; ++u) {
             sv[u] = (u < nu && lane + 64 * u < E) ? expf(sv[u] - zmax) : 0.f;
             zsum += sv[u];
         }
         zsum = wave_sum(zsum);
 #pragma unroll
-        for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+        for (int u = 0; u < NU; ++u) {
             const int e = lane + 64 * u;
             sv[u] = sv[u] / zsum;
             cv[u] = (u < nu && e < E) ? sv[u] + (correction ? correction[e] : 0.f) : -INFINITY;
@@ -130,21 +131,21 @@ __global__ __launch_bounds__(256) void moe_pick_grouped_kernel(const float* __re
             // A group is kept if fewer than keep_groups groups beat it (a larger score, or an equal one at a lower index).
             // Every lane learns the scores of its own outputs' groups, then counts the groups that beat them; what lies
             // outside the kept groups can no longer be chosen.
-            float own[MOE_MAX_EXPERTS / 64];
-            int beaten[MOE_MAX_EXPERTS / 64];
+            float own[NU];
+            int beaten[NU];
 #pragma unroll
-            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) { own[u] = -INFINITY; beaten[u] = 0; }
+            for (int u = 0; u < NU; ++u) { own[u] = -INFINITY; beaten[u] = 0; }
             for (int pass = 0; pass < 2; ++pass) {
                 for (int g = 0; g < n_groups; ++g) {
                     float m = -INFINITY;
 #pragma unroll
-                    for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+                    for (int u = 0; u < NU; ++u) {
                         const int e = lane + 64 * u;
                         if (u < nu && e < E && e / per == g) m = fmaxf(m, cv[u]);
                     }
                     m = wave_max(m);
 #pragma unroll
-                    for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+                    for (int u = 0; u < NU; ++u) {
                         const int mine = (lane + 64 * u) / per;
                         if (pass == 0) {
                             if (mine == g) own[u] = m;
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256) void moe_pick_grouped_kernel(const float* __re
                 }
             }
 #pragma unroll
-            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
+            for (int u = 0; u < NU; ++u)
                 if (beaten[u] >= keep_groups) cv[u] = -INFINITY;
         }
         int chosen[MOE_MAX_TOP];
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(256) void moe_pick_grouped_kernel(const float* __re
             float bz = -INFINITY;
             int best = 0x7fffffff;
 #pragma unroll
-            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u) {
+            for (int u = 0; u < NU; ++u) {
                 const int e = lane + 64 * u;
                 if (u < nu && e < E && cv[u] > -INFINITY && (cv[u] > bz || (cv[u] == bz && e < best))) { bz = cv[u]; best = e; }
             }
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(256) void moe_pick_grouped_kernel(const float* __re
             }
             float sw = 0.f;
 #pragma unroll
-            for (int u = 0; u < MOE_MAX_EXPERTS / 64; ++u)
+            for (int u = 0; u < NU; ++u)
                 if (u < nu && lane + 64 * u == best) { sw = sv[u]; cv[u] = -INFINITY; }      // taken
             sw = wave_sum(sw);                                     // (one lane holds it)
             chosen[k] = best;
@@ -279,8 +280,12 @@ extern "C" int fl_moe_route_grouped(const float* logits, int ld, int col0, int n
     }
     if (n == 0) return 0;
     const int pick_blocks = n < 4 * 1024 ? (n + 3) / 4 : 1024;
-    moe_pick_grouped_kernel<<<pick_blocks, 256, 0, stream>>>(logits, ld, col0, n, E, top, correction, n_groups, keep_groups, scale,
-                                                             place, pair_w);
+#define FL_PICK(NU) moe_pick_grouped_kernel<NU><<<pick_blocks, 256, 0, stream>>>(logits, ld, col0, n, E, top, correction, n_groups, keep_groups, scale, place, pair_w)
+    if (E <= 64) FL_PICK(1);               // (a lane's outputs live in registers: as few slots as the router's width needs)
+    else if (E <= 128) FL_PICK(2);
+    else if (E <= 256) FL_PICK(4);
+    else FL_PICK(MOE_MAX_EXPERTS / 64);
+#undef FL_PICK
     FL_LAUNCH_CHECK();
     moe_route_kernel<<<1, 1024, 0, stream>>>(n, E, E - n_identity, top, place, src_row, src_scale, pair_w, tiles, max_tiles);
     FL_LAUNCH_CHECK();

@@ -834,11 +834,13 @@ def channel_decay(a, col, a_log, dt_bias, out, n_heads, dim):
     return out
 
 
-def lowrank_expand(x, col, w, out):
-    """``out[t] = w @ x[t, col : col + rank]``: the second factor of a projection of low rank; ``x`` float32 rows (the
-    first factor's products, not rounded), ``w`` ``[features, rank]`` in its storage dtype, ``out`` float32."""
+def lowrank_expand(x, col, wt, out):
+    """``out[t] = wt.T @ x[t, col : col + rank]``: the second factor of a projection of low rank; ``x`` float32 rows (the
+    first factor's products, not rounded), ``wt`` the factor TRANSPOSED, ``[rank, features]``, in its storage dtype,
+    ``out`` float32."""
     n, ld = x.shape
-    N, R = w.shape
+    R, N = wt.shape
+    w = wt
     call("fl_lowrank_expand", _check(x, "lowrank_expand.x", torch.float32), ld, int(col), _check(w, "lowrank_expand.w"), dtype_code(w.dtype),
          _check(out, "lowrank_expand.out", torch.float32, (n, N)), n, N, R, stream_handle())
     return out

@@ -171,7 +171,8 @@ class GatedDelta(Mixer):
         self.col_b = self.channels
         self.col_a = self.col_b + H
         self.col_g = self.col_a + weights[a_name + ".weight"].shape[0]
-        self.w_a2, self.w_g2 = weights.get("a2.weight"), weights.get("g2.weight")     # (second factors: read row by row as they are stored)
+        # (second factors, transposed: the kernel that applies them reads neighbouring features side by side)
+        self.w_a2, self.w_g2 = (weights[k].t().contiguous() if k in weights else None for k in ("a2.weight", "g2.weight"))
         self.conv_w = torch.cat([weights[k + "_conv.weight"] for k in ("q", "k", "v")], dim=0).contiguous()
         self.a_log, self.dt_bias = weights["A_log"], weights["dt_bias"]
         self.norm = weights["norm.weight"].repeat(H).contiguous()          # one gain for every head, laid out heads x vdim
