@@ -327,9 +327,10 @@ int fl_linear_scan_delta_channel(const float* q, int ldq, const float* k, int ld
 // out[t][h * D + d] = exp(-exp(a_log[h]) * softplus(a[t][col + h * D + d] + dt_bias[h * D + d]))
 int fl_channel_decay(const float* a, int ld, int col, const float* a_log, const float* dt_bias, float* out,
                      int n, int H, int D, hipStream_t stream);
-// out[t][f] = sum_r x[t][col + r] * wt[r][f]: the second factor of a projection of low rank, transposed (x float, wt in dtype)
-int fl_lowrank_expand(const float* x, int ld, int col, const void* w, int dtype, float* out, int n, int N, int R,
-                      hipStream_t stream);
+// out[t][f] = sum_r x[t][col + r] * w[f][r]: the second factor of a projection of low rank, given as it is stored
+// (w_rows [N][R]: a step of few tokens reads it) and transposed (wt [R][N]); x float, the factor in dtype
+int fl_lowrank_expand(const float* x, int ld, int col, const void* w_rows, const void* wt, int dtype, float* out,
+                      int n, int N, int R, hipStream_t stream);
 int fl_rotate_scale(const float* proj, int ld, int col_a, int col_b, const float* cs, int rot, int interleaved,
                     float scale_a, float scale_b, float* out_a, float* out_b, int n, int H, int D,
                     hipStream_t stream);

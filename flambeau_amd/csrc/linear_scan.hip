@@ -255,28 +255,69 @@ FL_RECORDABLE(fl_channel_decay)
 // out[t][f] = sum_r x[t][col + r] * wt[r][f] for a short run of r (the second factor of a projection of low rank, given
 // TRANSPOSED, [rank][features], so that neighbouring threads read neighbouring values): x float rows, wt in its
 // storage type, float sums in rising order of r
+#define LR_TOKENS 8           // tokens a block of fl_lowrank_expand takes: a value of wt is read once for all of them
+#define LR_FEW 16             // up to this many tokens a thread reads its feature's own row of the factor as it is stored
+// (a step of few tokens: a block per token and 256 features, a thread walks the R neighbouring values of its feature's
+// row, which the compiler fetches some at a time; the sums run in rising order of r as in the kernel below)
 template <typename T>
-__global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __restrict__ x, int ld, int col, const T* __restrict__ w,
-                                                             float* __restrict__ out, int N, int R) {
+__global__ __launch_bounds__(256) void lowrank_expand_rows_kernel(const float* __restrict__ x, int ld, int col, const T* __restrict__ w,
+                                                                  float* __restrict__ out, int N, int R) {
     extern __shared__ float xr[];
     const int t = blockIdx.y;
     for (int r = threadIdx.x; r < R; r += 256) xr[r] = x[(size_t)t * ld + col + r];
     __syncthreads();
     const int f = blockIdx.x * 256 + threadIdx.x;
     if (f >= N) return;
+    const T* wr = w + (size_t)f * R;
     float s = 0.f;
-    for (int r = 0; r < R; ++r) s = fmaf(xr[r], to_f32(w[(size_t)r * N + f]), s);
+    for (int r = 0; r < R; ++r) s = fmaf(xr[r], to_f32(wr[r]), s);
     out[(size_t)t * N + f] = s;
 }
 
-extern "C" int fl_lowrank_expand(const float* x, int ld, int col, const void* w, int dtype, float* out, int n, int N, int R,
-                                 hipStream_t stream) {
-    FL_CHECK(n >= 0 && N > 0 && R > 0 && R <= 4096 && col >= 0 && ld >= col + R, "lowrank_expand: columns %d..%d of rows %d wide", col, col + R, ld);
+template <typename T>
+__global__ __launch_bounds__(256) void lowrank_expand_kernel(const float* __restrict__ x, int ld, int col, const T* __restrict__ w,
+                                                             float* __restrict__ out, int n, int N, int R) {
+    extern __shared__ float xr[];                         // [LR_TOKENS][R]
+    const int t0 = blockIdx.y * LR_TOKENS, cnt = min(LR_TOKENS, n - t0);
+    for (int e = threadIdx.x; e < LR_TOKENS * R; e += 256) {
+        const int tt = e / R, r = e - tt * R;
+        xr[e] = tt < cnt ? x[(size_t)(t0 + tt) * ld + col + r] : 0.f;
+    }
+    __syncthreads();
+    const int f = blockIdx.x * 256 + threadIdx.x;
+    if (f >= N) return;
+    float s[LR_TOKENS];
+#pragma unroll
+    for (int tt = 0; tt < LR_TOKENS; ++tt) s[tt] = 0.f;
+#pragma unroll 8
+    for (int r = 0; r < R; ++r) {
+        const float wv = to_f32(w[(size_t)r * N + f]);
+#pragma unroll
+        for (int tt = 0; tt < LR_TOKENS; ++tt) s[tt] = fmaf(xr[tt * R + r], wv, s[tt]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < LR_TOKENS; ++tt)
+        if (tt < cnt) out[(size_t)(t0 + tt) * N + f] = s[tt];
+}
+
+extern "C" int fl_lowrank_expand(const float* x, int ld, int col, const void* w_rows, const void* w, int dtype, float* out,
+                                 int n, int N, int R, hipStream_t stream) {
+    FL_CHECK(n >= 0 && N > 0 && R > 0 && R <= 1024 && col >= 0 && ld >= col + R, "lowrank_expand: columns %d..%d of rows %d wide (a rank of at most 1024)", col, col + R, ld);
+    FL_CHECK(w_rows && w, "lowrank_expand: the factor is wanted as it is stored and transposed");
     if (n == 0) return 0;
-    FL_CHECK(n <= 65535, "lowrank_expand: %d rows are more than one grid takes", n);
-    dim3 grid(ceil_div(N, 256), n);
-    if (dtype == FL_F32) lowrank_expand_kernel<float><<<grid, 256, R * sizeof(float), stream>>>(x, ld, col, (const float*)w, out, N, R);
-    else if (dtype == FL_BF16) lowrank_expand_kernel<bf16_t><<<grid, 256, R * sizeof(float), stream>>>(x, ld, col, (const bf16_t*)w, out, N, R);
+    if (n <= LR_FEW) {
+        dim3 grid(ceil_div(N, 256), n);
+        if (dtype == FL_F32) lowrank_expand_rows_kernel<float><<<grid, 256, R * sizeof(float), stream>>>(x, ld, col, (const float*)w_rows, out, N, R);
+        else if (dtype == FL_BF16) lowrank_expand_rows_kernel<bf16_t><<<grid, 256, R * sizeof(float), stream>>>(x, ld, col, (const bf16_t*)w_rows, out, N, R);
+        else FL_CHECK(false, "lowrank_expand: unknown dtype %d", dtype);
+        FL_LAUNCH_CHECK();
+        return 0;
+    }
+    dim3 grid(ceil_div(N, 256), ceil_div(n, LR_TOKENS));
+    FL_CHECK(grid.y <= 65535, "lowrank_expand: %d rows are more than one grid takes", n);
+    const size_t lds = (size_t)LR_TOKENS * R * sizeof(float);
+    if (dtype == FL_F32) lowrank_expand_kernel<float><<<grid, 256, lds, stream>>>(x, ld, col, (const float*)w, out, n, N, R);
+    else if (dtype == FL_BF16) lowrank_expand_kernel<bf16_t><<<grid, 256, lds, stream>>>(x, ld, col, (const bf16_t*)w, out, n, N, R);
     else FL_CHECK(false, "lowrank_expand: unknown dtype %d", dtype);
     FL_LAUNCH_CHECK();
     return 0;

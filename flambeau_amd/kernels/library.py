@@ -72,7 +72,7 @@ _SIGNATURES = {
     "fl_attn_mixed_tiled": [P, P, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, I, I, P, P, P, I, I, P, P, P],
     "fl_linear_scan_delta_channel": [P, I, P, I, P, I, P, I, P, I, P, L, P, P, P, P, I, I, I, I, I, P],
     "fl_channel_decay": [P, I, I, P, P, P, I, I, I, P],
-    "fl_lowrank_expand": [P, I, I, P, I, P, I, I, I, P],
+    "fl_lowrank_expand": [P, I, I, P, P, I, P, I, I, I, P],
     "fl_moe_route_grouped": [P, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, I, P],
     "fl_moe_identity": [P, I, P, P, P, P, I, I, P],
     "fl_hyper_step": [P, I, I, I, P, P, P, P, P, I, P, P, F, P, I, P],

@@ -834,14 +834,15 @@ def channel_decay(a, col, a_log, dt_bias, out, n_heads, dim):
     return out
 
 
-def lowrank_expand(x, col, wt, out):
-    """``out[t] = wt.T @ x[t, col : col + rank]``: the second factor of a projection of low rank; ``x`` float32 rows (the
-    first factor's products, not rounded), ``wt`` the factor TRANSPOSED, ``[rank, features]``, in its storage dtype,
-    ``out`` float32."""
+def lowrank_expand(x, col, w, wt, out):
+    """``out[t] = w @ x[t, col : col + rank]``: the second factor of a projection of low rank; ``x`` float32 rows (the
+    first factor's products, not rounded), ``w`` the factor ``[features, rank]`` as it is stored and ``wt`` the same
+    transposed (a step of few tokens reads the one, a larger step the other: the same sums in the same order), ``out`` float32."""
     n, ld = x.shape
-    R, N = wt.shape
-    w = wt
-    call("fl_lowrank_expand", _check(x, "lowrank_expand.x", torch.float32), ld, int(col), _check(w, "lowrank_expand.w"), dtype_code(w.dtype),
+    N, R = w.shape
+    if wt.shape != (R, N) or wt.dtype != w.dtype:
+        raise KernelError(f"lowrank_expand: a factor {tuple(w.shape)} with a transposed copy {tuple(wt.shape)}")
+    call("fl_lowrank_expand", _check(x, "lowrank_expand.x", torch.float32), ld, int(col), _check(w, "lowrank_expand.w"), _check(wt, "lowrank_expand.wt"), dtype_code(w.dtype),
          _check(out, "lowrank_expand.out", torch.float32, (n, N)), n, N, R, stream_handle())
     return out
 

@@ -171,8 +171,9 @@ class GatedDelta(Mixer):
         self.col_b = self.channels
         self.col_a = self.col_b + H
         self.col_g = self.col_a + weights[a_name + ".weight"].shape[0]
-        # (second factors, transposed: the kernel that applies them reads neighbouring features side by side)
-        self.w_a2, self.w_g2 = (weights[k].t().contiguous() if k in weights else None for k in ("a2.weight", "g2.weight"))
+        # (second factors, as they are stored and transposed: a step of few tokens reads a feature's own row, a larger one
+        # neighbouring features side by side)
+        self.w_a2, self.w_g2 = ((weights[k].contiguous(), weights[k].t().contiguous()) if k in weights else None for k in ("a2.weight", "g2.weight"))
         self.conv_w = torch.cat([weights[k + "_conv.weight"] for k in ("q", "k", "v")], dim=0).contiguous()
         self.a_log, self.dt_bias = weights["A_log"], weights["dt_bias"]
         self.norm = weights["norm.weight"].repeat(H).contiguous()          # one gain for every head, laid out heads x vdim
@@ -195,14 +196,14 @@ class GatedDelta(Mixer):
             # projection or through the second factor of a projection of low rank (its first factor's products in 32-bit)
             a, col = proj, self.col_a
             if self.w_a2 is not None:
-                a, col = ops.lowrank_expand(proj, self.col_a, self.w_a2, rt.buffer("gd_decay_in", n, H * D, torch.float32)), 0
+                a, col = ops.lowrank_expand(proj, self.col_a, *self.w_a2, rt.buffer("gd_decay_in", n, H * D, torch.float32)), 0
             key_decay = ops.channel_decay(a, col, self.a_log, self.dt_bias, rt.buffer("gd_decay", n, H * D, torch.float32), H, D)
         hidden = rt.buffer("gd_hidden", n, H * Dv, torch.float32)
         ops.linear_scan(prep[:, :G * D], prep[:, G * D:2 * G * D], prep[:, 2 * G * D:], cache.state, step.seq_q_start,
                         step.seq_q_len, step.seq_slots, hidden, H, G, D, Dv, token_gates=gates, key_decay=key_decay)
         gate_rows, gate_col = proj, self.col_g
         if self.w_g2 is not None:
-            gate_rows, gate_col = ops.lowrank_expand(proj, self.col_g, self.w_g2, rt.buffer("gd_gate_in", n, H * Dv, torch.float32)), 0
+            gate_rows, gate_col = ops.lowrank_expand(proj, self.col_g, *self.w_g2, rt.buffer("gd_gate_in", n, H * Dv, torch.float32)), 0
         out = rt.buffer("gd_out", n, H * Dv)
         ops.headnorm_gate(hidden, self.norm, gate_rows, gate_col, out, H, self.eps, gate_kind=self.gate)
         return Product(out, self.w_o)
