@@ -81,7 +81,7 @@ def _feed_forward(cfg: LenedraConfig, f, p: str):
 
 def lenedra_spec(cfg: LenedraConfig) -> ModelSpec:
     norm = PartSpec("rmsnorm", dict(hidden_size=cfg.width, eps=cfg.eps, unit_offset=True))
-    layers, run_order = [], []
+    layers, run_order, unread = [], [], []
     for l, layer in enumerate(cfg.layers):
         p = f"l{l}."
         mixer, names = _mixer(cfg, l)
@@ -99,6 +99,8 @@ def lenedra_spec(cfg: LenedraConfig) -> ModelSpec:
             block = PartSpec("prenorm", dict(mixer=mixer, feed_forward=ffn, norm=norm))
         layers.append(LayerSpec(block, names))
         run_order.append(RunEntry(l))
+        if ffn is None:                         # (a file may still hold the second sublayer's norm and numbers: nothing reads them)
+            unread += [f"{p}norm2", f"{p}hc2.*"]
     return ModelSpec(
         architecture=cfg.architecture,
         hidden_size=cfg.width,
@@ -114,6 +116,7 @@ def lenedra_spec(cfg: LenedraConfig) -> ModelSpec:
         embedding=PartSpec("scaled_token_embedding", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.width, scale=cfg.embedding_scale)),
         head=PartSpec("capped_linear_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.width, softcap=cfg.logit_softcap)),
         residual_streams=cfg.streams,
+        ignored_tensors=tuple(unread),
     )
 
 
