@@ -5,7 +5,7 @@ A pre-norm decoder whose residual stream is kept in several copies (hyper-connec
 with the weight stored around zero, behind an embedding that is multiplied by a constant and in front of a head whose
 logits pass a soft cap.  Mixers, layer by layer as config.json lists them:
 
-* ``attention``: ``mixed_heads_attention`` with biased projections, values that are the keys as projected, a norm per
+* ``attention``: ``mixed_heads_attention`` with biased projections, no value projection (a key's raw projection is also its value), a norm per
   head with a gain shared by the heads, a distance bias with slopes 2^(-8 (h + 1) / heads), a sliding window beside
   which the first tokens stay visible, a biased output projection;
 * ``parallel``: ``side_by_side`` (no norms, a factor each) of ``mixed_heads_attention`` with biased projections, a

@@ -251,8 +251,8 @@ class MixedHeadsAttention(NormedGQAAttention):
       visible to every later query beside the window (at their true positions); ``chunk`` > 0 instead of a window: a
       query sees the earlier keys of its own run of ``chunk`` positions, counted from position 0 of the sequence;
     * ``bias``: the projections of q, k and v have biases; ``out_bias``: the output projection has one;
-    * ``values="keys"``: there is no value projection, the values are the keys as projected (bias included, before
-      their norm); key and value size are then equal.
+    * ``values="keys"``: there is no value projection: what the key projection returns for a token (bias included, ahead of
+      the keys' norm) is also that token's value; key and value size are then equal.
 
     ``own_kv=False``: the layer has no key and value projections (nor their norm); its run-order entry reads the
     cache of an earlier entry with equal head counts and sizes.  ``cache_window``: how many of the newest keys the

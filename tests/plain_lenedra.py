@@ -96,7 +96,7 @@ def softmax_attention(q, k, v, mask, scale, slopes=None, sink=None):
 
 # ---------------------------------------------------------------- mixers
 def attention(h, m, t, p, eps):
-    """Keys double as values (as projected, before their norm); q and k normed per head with a gain shared by
+    """What the key projection returns is used twice: raw as the value, normed as the key; q and k normed per head with a gain shared by
     the heads; a distance bias; a sliding window that also keeps the first tokens."""
     T = h.shape[0]
     H, G, D = m["heads"], m["kv_heads"], m["dim"]
