@@ -310,6 +310,7 @@ FL_RECORDABLE(fl_attn_mixed)
 //      the (head, half chunk) tiles are dealt out to the waves, operands come straight from q and the pages
 //   2. score[h][pair] = sum_g talk[h][g] * raw[g][pair]                v_mfma_f32_16x16x4_f32 (true 32-bit): the
 //      mixing matrix is the A operand, 16 (query, key) pairs are a B operand's columns, both read from LDS
+//      (left out, with its barrier, where there is no mixing matrix: phase 1 then writes the scores where phase 3 reads)
 //   3. a thread per (head, query) row: mask, running maximum and sum (they stay in that thread's registers from
 //      chunk to chunk), weights as bfloat16 into LDS, and the factor by which the row's output shrinks
 //   4. out[h][query][:] = factor * out + P_h . V                        v_mfma_f32_16x16x32_bf16; a wave owns up to four
@@ -398,6 +399,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
         return;
     }
     const int group = nh / cache.n_kv_heads;
+    const bool mixes = a.talk != nullptr;              // (the same for every block: a mixing matrix, or every head for itself)
     const bf16_t* kv = (const bf16_t*)cache.base;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
@@ -485,13 +487,17 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int qq = 4 * lg + r;
-                        raw[g * AT_RAW_LD + qq * AT_RAW_Q + 16 * kt + li] = acc[r] * a.scale - slope * (float)(p_first + qq - jpos[kt]);
+                        const float sv = acc[r] * a.scale - slope * (float)(p_first + qq - jpos[kt]);
+                        // (without a mixing matrix a head's score is its own raw score: it goes where phase 3 reads, and phase 2 is left out)
+                        if (mixes) raw[g * AT_RAW_LD + qq * AT_RAW_Q + 16 * kt + li] = sv;
+                        else sc[g * AT_SC_LD + qq * (AT_CHUNK + 1) + 16 * kt + li] = sv;
                     }
                 }
             }
         }
         __syncthreads();
         // ---- 2. the heads' scores mixed: 16 pairs at a time, pairs of the queries that exist
+        if (mixes) {
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
             if (16 * hb >= HP) continue;
@@ -509,6 +515,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_mixed_tiled_kernel(const bf16
             }
         }
         __syncthreads();
+        }
         // ---- 3. the rows' softmax.  Most chunks lie inside every row's window: there no key is tested
         if (rh < nh) {
             u32x4* prow4 = (u32x4*)(pb + (rh * AT_ROWS + rq) * AT_P_LD);      // eight weights a store
