@@ -303,8 +303,8 @@ int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, int col_v, c
                    const int* tok_seq, const int* block_table, int max_blocks, void* q_out, void* cache_base,
                    int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
                    int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
-                   const float* q_head_gain, const float* k_head_gain, float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
-                   float* row_scales, hipStream_t stream);
+                   const float* q_head_gain, const float* k_head_gain, float eps, float* v_first, int vmix_mode,
+                   const float* lambda, int write_cache, float* row_scales, const float* bias, hipStream_t stream);
 
 // ---- linear recurrences with a matrix state per head (linear_scan.hip) ----
 int fl_linear_scan_max_dim(void);
@@ -375,10 +375,10 @@ int fl_attn_mixed_tiled(const void* q, void* out, const void* cache_base, const 
                         hipStream_t stream);
 
 // ---- hyper-connections: a residual stream in S copies (hyper.hip) ----
-// xs [n][S][W] float.  y given: x_t <- sum_s mix[s][t] x_s + out_w[t] * y.  in_w given: u = sum_s in_w[s] x_s (the new
+// xs [n][S][W] float.  y given: x_t <- sum_s mix[s][t] x_s + out_w[t] * (y + y_bias), y_bias [W] or null.  in_w given: u = sum_s in_w[s] x_s (the new
 // copies) into u_out, and with a gain normed = u / sqrt(mean(u^2) + eps) * gain in out_dtype.  rows (n_rows of them):
 // the tokens that are read, one output row each (only without y).
-int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* mix, const float* out_w,
+int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* y_bias, const float* mix, const float* out_w,
                   const float* in_w, const int* rows, int n_rows, float* u_out, const float* gain, float eps,
                   void* normed, int out_dtype, hipStream_t stream);
 int fl_hyper_spread(const float* x, float* xs, int n, int S, int W, hipStream_t stream);

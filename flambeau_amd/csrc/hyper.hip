@@ -4,6 +4,7 @@
 // in[S], out[S] and mix[S][S] (indexed [from][to]):
 //     u   = sum_s in[s] x_s                      what the sublayer's norm reads
 //     x_t <- sum_s mix[s][t] x_s + out[t] * y    all copies at once from the old ones, y the sublayer's output
+//                                                (plus y_bias, one value per column, where the sublayer's last product has a bias)
 // fl_hyper_step does the second line for the sublayer that has just run (if y is given) and the first for the one
 // that runs next (if `in` is given), in one pass over the copies: the new copies are written, their weighted sum u is
 // kept in float (u_out) and, if a gain is given, normed in the same kernel:
@@ -21,6 +22,7 @@
 struct HyperStep {
     float* xs; int S, W;
     const float* y;                 // [n][W] or null: nothing is written
+    const float* y_bias;            // [W] or null: added to every row of y as it is read (a bias of the sublayer's last product)
     const float* mix; const float* out_w;
     const float* in_w;              // [S] or null: nothing is read
     float* u_out;                   // [n][W] or null
@@ -62,7 +64,8 @@ __global__ __launch_bounds__(NT) void hyper_step_kernel(HyperStep a, T* __restri
             if (s < S) old[s] = *(const vec_t*)(x + (size_t)s * W + c);
         vec_t u = 0.f;
         if (yr) {
-            const vec_t yv = *(const vec_t*)(yr + c);
+            vec_t yv = *(const vec_t*)(yr + c);
+            if (a.y_bias) yv += *(const vec_t*)(a.y_bias + c);
 #pragma unroll
             for (int to = 0; to < SMAX; ++to) {
                 if (to >= S) break;
@@ -115,17 +118,18 @@ __global__ __launch_bounds__(NT) void hyper_step_kernel(HyperStep a, T* __restri
 
 #define HY_WIDE_ROW 2048      // from this many values a row a block has 1,024 threads
 
-extern "C" int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* mix, const float* out_w,
+extern "C" int fl_hyper_step(float* xs, int n, int S, int W, const float* y, const float* y_bias, const float* mix, const float* out_w,
                              const float* in_w, const int* rows, int n_rows, float* u_out, const float* gain, float eps,
                              void* normed, int out_dtype, hipStream_t stream) {
     FL_CHECK(n >= 0 && S >= 1 && S <= HY_MAX_STREAMS && W > 0, "hyper_step: %d copies of %d values (at most %d copies)", S, W, HY_MAX_STREAMS);
     FL_CHECK(!y || (mix && out_w), "hyper_step: a sublayer's output without its numbers");
+    FL_CHECK(y || !y_bias, "hyper_step: a bias without the output it belongs to");
     FL_CHECK(!gain || (in_w && u_out && normed), "hyper_step: a norm needs what it reads and where it writes");
     FL_CHECK(!rows || !y, "hyper_step: picked rows are read only");
     FL_CHECK(out_dtype == FL_F32 || out_dtype == FL_BF16, "hyper_step: unknown dtype %d", out_dtype);
     const int blocks = rows ? n_rows : n;
     if (blocks <= 0) return 0;
-    HyperStep a{xs, S, W, y, mix, out_w, in_w, u_out, gain, eps, rows};
+    HyperStep a{xs, S, W, y, y_bias, mix, out_w, in_w, u_out, gain, eps, rows};
     const bool few = W >= HY_WIDE_ROW, wide = W % 4 == 0, small = S <= 4;
 #define FL_HY(T, NT, VEC, KEEP, SMAX) hyper_step_kernel<T, NT, VEC, KEEP, SMAX><<<blocks, NT, 0, stream>>>(a, (T*)normed)
 #define FL_HY_S(T, NT, VEC, KEEP) do { if (small) FL_HY(T, NT, VEC, KEEP, 4); else FL_HY(T, NT, VEC, KEEP, HY_MAX_STREAMS); } while (0)

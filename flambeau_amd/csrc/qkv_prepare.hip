@@ -8,7 +8,8 @@
 //     head dim that all heads of q (of k) share, or not;
 //   * values blended with those an earlier layer made for the same token,
 //     v <- (1 - lambda) v + lambda v_first, or kept as that first layer's for later ones;
-//   * q stored for the attention kernels, k and v stored into the paged cache at the token's position.
+//   * q stored for the attention kernels, k and v stored into the paged cache at the token's position;
+//   * ahead of all of it, the projections' biases (one value per column of the joined projection), or none.
 // Heads are stored `hdp` wide (hdp >= max(D, Dv)): keys are padded with zeros behind D, values behind
 // Dv, queries behind D, so that attention kernels of one head size serve key and value sizes that differ.
 // The projection arrives in float; everything here is float, only the stores are in the cache's type.
@@ -28,15 +29,17 @@ struct QkvPrepare {
     float* v_first; int vmix_mode; const float* lambda;
     int write_cache;
     float* row_scales;          // [n][2]: 1 / rms of every token's q and k projection, made by a kernel of its own (or null)
+    const float* bias;          // [ld] or null: added to the projection's columns as they are read
 };
 
 // The norm over the whole projection of q and of k: 1 / sqrt(mean(x^2) + eps) of both for one token per block.
 __global__ __launch_bounds__(256) void qkv_row_scales_kernel(QkvPrepare a, int nkv) {
     __shared__ float lds[8];
     const float* row = a.proj + (size_t)blockIdx.x * a.ld;
+    auto at = [&](int c) { return a.bias ? row[c] + a.bias[c] : row[c]; };
     float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < a.nh * a.D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
-    if (a.col_k >= 0) for (int i = threadIdx.x; i < nkv * a.D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
+    for (int i = threadIdx.x; i < a.nh * a.D; i += 256) sq = fmaf(at(a.col_q + i), at(a.col_q + i), sq);
+    if (a.col_k >= 0) for (int i = threadIdx.x; i < nkv * a.D; i += 256) sk = fmaf(at(a.col_k + i), at(a.col_k + i), sk);
     sq = block_sum<4>(sq, lds);
     sk = block_sum<4>(sk, lds + 4);
     if (threadIdx.x == 0) {
@@ -51,6 +54,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     const int token = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nh = a.nh, nkv = cache.n_kv_heads, D = a.D, Dv = a.Dv, hdp = a.hdp;
     const float* row = a.proj + (size_t)token * a.ld;
+    auto at = [&](int c) { return a.bias ? row[c] + a.bias[c] : row[c]; };       // a column of the projection, its bias added
     const bool has_kv = a.col_k >= 0;                 // (a mixer that reads another layer's keys and values projects queries alone)
     float inv_q = 1.f, inv_k = 1.f;
     if (a.qnorm_w && a.row_scales) {
@@ -59,8 +63,8 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     } else if (a.qnorm_w) {
         // (a step of few tokens: every block sums for itself, in the same order as the kernel above, and a launch is saved)
         float sq = 0.f, sk = 0.f;
-        for (int i = threadIdx.x; i < nh * D; i += 256) sq = fmaf(row[a.col_q + i], row[a.col_q + i], sq);
-        if (has_kv) for (int i = threadIdx.x; i < nkv * D; i += 256) sk = fmaf(row[a.col_k + i], row[a.col_k + i], sk);
+        for (int i = threadIdx.x; i < nh * D; i += 256) sq = fmaf(at(a.col_q + i), at(a.col_q + i), sq);
+        if (has_kv) for (int i = threadIdx.x; i < nkv * D; i += 256) sk = fmaf(at(a.col_k + i), at(a.col_k + i), sk);
         inv_q = 1.0f / sqrtf(block_sum<4>(sq, lds) / (float)(nh * D) + a.eps);
         inv_k = 1.0f / sqrtf(block_sum<4>(sk, lds + 4) / (float)(nkv * D) + a.eps);
     }
@@ -78,10 +82,10 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
     if (head < nh + (has_kv ? nkv : 0)) {
         const bool is_q = head < nh;
         const int h = is_q ? head : head - nh;
-        const float* src = row + (is_q ? a.col_q : a.col_k) + h * D;
+        const int src = (is_q ? a.col_q : a.col_k) + h * D;
         const float* gain = is_q ? a.qnorm_w : a.knorm_w;
         const float inv = is_q ? inv_q : inv_k;
-        auto value = [&](int d) { return gain ? src[d] * inv * gain[h * D + d] : src[d]; };
+        auto value = [&](int d) { return gain ? at(src + d) * inv * gain[h * D + d] : at(src + d); };
         float r[4];
         float ss = 0.f;
 #pragma unroll
@@ -126,7 +130,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(QkvPrepare a, T* __res
         const int h = e / hdp, d = e - h * hdp;
         float v = 0.f;
         if (d < Dv) {
-            v = row[a.col_v + h * Dv + d];
+            v = at(a.col_v + h * Dv + d);
             const size_t at = (size_t)token * nkv * Dv + h * Dv + d;
             if (a.vmix_mode == 1) a.v_first[at] = v;
             else if (a.vmix_mode == 2) v = (1.0f - lam) * v + lam * a.v_first[at];
@@ -140,7 +144,7 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
                               int dtype, int n, int nh, int nkv, int D, int Dv, int hdp, int page_size, int n_pages, int rot,
                               int interleaved, const float* cs, const float* qnorm_w, const float* knorm_w, int head_norm,
                               const float* q_head_gain, const float* k_head_gain, float eps, float* v_first, int vmix_mode, const float* lambda, int write_cache,
-                              float* row_scales, hipStream_t stream) {
+                              float* row_scales, const float* bias, hipStream_t stream) {
     FL_CHECK(n >= 0 && nh > 0 && nkv > 0 && D > 0 && Dv > 0 && page_size > 0, "qkv_prepare: bad sizes");
     FL_CHECK(hdp >= D && hdp >= Dv && hdp <= 256, "qkv_prepare: heads of %d and %d values stored %d wide (at most 256)", D, Dv, hdp);
     FL_CHECK(rot >= 0 && rot <= D && rot % 2 == 0, "qkv_prepare: rotated dims %d of head %d", rot, D);
@@ -154,7 +158,7 @@ extern "C" int fl_qkv_prepare(const float* proj, int ld, int col_q, int col_k, i
     if (n == 0) return 0;
     QkvPrepare a{proj, ld, col_q, col_k, col_v, positions, tok_seq, block_table, max_blocks, nh, D, Dv, hdp,
                  rot, interleaved, (const float2*)cs, qnorm_w, knorm_w, head_norm, eps, q_head_gain, k_head_gain, v_first, vmix_mode, lambda, write_cache,
-                 (qnorm_w && n > QKV_FEW_TOKENS) ? row_scales : nullptr};
+                 (qnorm_w && n > QKV_FEW_TOKENS) ? row_scales : nullptr, bias};
     PagedCache c{cache_base, nkv, page_size, hdp, n_pages};
     dim3 grid(n, ceil_div(nh + (col_k >= 0 ? nkv : 0), 4));
     FL_CHECK(grid.y <= 65535, "qkv_prepare: %d heads are more than one grid takes", nh + nkv);

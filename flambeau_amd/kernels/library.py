@@ -56,7 +56,7 @@ _SIGNATURES = {
     "fl_gated_act": [P, P, I, I, I, I, P],
     "fl_norm_mix": [P, P, F, P, P, F, P, I, I, F, P],
     "fl_heads_gate": [P, I, I, P, I, I, I, P, I, I, I, P],
-    "fl_qkv_prepare": [P, I, I, I, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, I, I, I, P, P, P, I, P, P, F, P, I, P, I, P, P],
+    "fl_qkv_prepare": [P, I, I, I, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, I, I, I, P, P, P, I, P, P, F, P, I, P, I, P, P, P],
     "fl_linear_scan": [P, I, P, I, P, I, P, P, P, I, P, L, P, P, P, P, I, I, I, I, I, P],
     "fl_conv_prepare": [P, I, I, I, I, P, P, P, P, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, P],
     "fl_rotate_scale": [P, I, I, I, P, I, I, F, F, P, P, I, I, I, P],
@@ -75,7 +75,7 @@ _SIGNATURES = {
     "fl_lowrank_expand": [P, I, I, P, P, I, P, I, I, I, P],
     "fl_moe_route_grouped": [P, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, I, P],
     "fl_moe_identity": [P, I, P, P, P, P, I, I, P],
-    "fl_hyper_step": [P, I, I, I, P, P, P, P, P, I, P, P, F, P, I, P],
+    "fl_hyper_step": [P, I, I, I, P, P, P, P, P, P, I, P, P, F, P, I, P],
     "fl_hyper_spread": [P, P, I, I, I, P],
     "fl_scaled_sum": [P, F, P, F, P, L, P],
     "fl_softcap_inplace": [P, L, F, P],

@@ -569,12 +569,13 @@ def heads_gate(x, head_stride, gate, gate_col0, kind, out, n_heads):
 
 def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: PagedLayerCache, n_heads, dim, vdim, rotated_dims,
                 interleaved, table, q_gain, k_gain, head_norm, eps, v_first=None, value_mix: int = 0, mix=None, write_cache=True,
-                row_scales=None, q_head_gain=None, k_head_gain=None):
+                row_scales=None, q_head_gain=None, k_head_gain=None, bias=None):
     """From the float32 rows of a joined projection (q, k, v at the columns ``cols``) to the rotated, normed
     queries in ``q_out`` and the token's keys and values in the cache, heads stored ``cache.head_dim`` wide.
     ``q_gain`` / ``k_gain``: gains of a norm over the whole projection of q and of k (before rotation);
     ``head_norm``: every head divided by its root mean square after rotation, times ``q_head_gain`` / ``k_head_gain``
-    (float32 ``[dim]``, one gain per head dim that all heads share) where given; ``value_mix``: 1 keeps the
+    (float32 ``[dim]``, one gain per head dim that all heads share) where given; ``bias``: float32, one value per column of
+    ``proj``, added to the projection as it is read (the projections' biases); ``value_mix``: 1 keeps the
     values in ``v_first``, 2 blends them with it by the device scalar ``mix``; ``row_scales``: float32 ``[n, 2]`` of
     scratch for the norm over the projection (a step of many tokens forms its sums in a kernel of their own)."""
     n, ld = proj.shape
@@ -596,7 +597,8 @@ def qkv_prepare(proj, cols, positions, tok_seq, block_table, q_out, cache: Paged
          _check(k_head_gain, "qkv_prepare.k_head_gain", torch.float32, (dim,)) if k_head_gain is not None else None, float(eps),
          _check(v_first, "qkv_prepare.v_first", torch.float32, (n, nkv * vdim)) if v_first is not None else None, int(value_mix),
          _check(mix, "qkv_prepare.mix", torch.float32) if mix is not None else None, int(bool(write_cache)),
-         _check(row_scales, "qkv_prepare.row_scales", torch.float32, (n, 2)) if row_scales is not None else None, stream_handle())
+         _check(row_scales, "qkv_prepare.row_scales", torch.float32, (n, 2)) if row_scales is not None else None,
+         _check(bias, "qkv_prepare.bias", torch.float32, (ld,)) if bias is not None else None, stream_handle())
     return q_out
 
 
@@ -883,16 +885,17 @@ def hyper_spread(x, xs, n_streams):
     return xs
 
 
-def hyper_step(xs, n_streams, y=None, mix=None, out_w=None, in_w=None, u_out=None, gain=None, eps=0.0, normed=None, rows=None):
+def hyper_step(xs, n_streams, y=None, mix=None, out_w=None, in_w=None, u_out=None, gain=None, eps=0.0, normed=None, rows=None,
+               y_bias=None):
     """One pass over the copies ``xs`` float32 ``[n, S * W]`` of a stream.  With ``y`` (float32 ``[n, W]``, a sublayer's
-    output): x_t <- sum_s mix[s, t] x_s + out_w[t] y.  With ``in_w``: u = sum_s in_w[s] x_s of the new copies into ``u_out``
+    output, plus ``y_bias`` float32 ``[W]`` in every row where given): x_t <- sum_s mix[s, t] x_s + out_w[t] y.  With ``in_w``: u = sum_s in_w[s] x_s of the new copies into ``u_out``
     and, with ``gain``, ``normed = u / sqrt(mean(u^2) + eps) * gain``.  ``rows`` (int32) picks the tokens that are read."""
     n, SW = xs.shape
     S = int(n_streams)
     W = SW // S
     f = lambda t, name, shape: _check(t, "hyper_step." + name, torch.float32, shape) if t is not None else None
     n_rows = rows.shape[0] if rows is not None else n
-    call("fl_hyper_step", _check(xs, "hyper_step.xs", torch.float32), n, S, W, f(y, "y", (n, W)), f(mix, "mix", (S, S)),
+    call("fl_hyper_step", _check(xs, "hyper_step.xs", torch.float32), n, S, W, f(y, "y", (n, W)), f(y_bias, "y_bias", (W,)), f(mix, "mix", (S, S)),
          f(out_w, "out", (S,)), f(in_w, "in", (S,)), _check(rows, "hyper_step.rows", torch.int32) if rows is not None else None, n_rows,
          f(u_out, "u", (n_rows, W)), f(gain, "gain", (W,)), float(eps),
          _check(normed, "hyper_step.normed", None, (n_rows, W)) if normed is not None else None,

@@ -20,7 +20,7 @@ from ..config.base import ConfigError
 from ..kernels import ops
 from ..kernels import paged_attention  # noqa: F401  (registers this mixer's kernel set)
 from ..kernels import mixed_attention  # noqa: F401  (the kernel set of attention whose heads' scores are mixed)
-from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedKVSpec, PartSpec, Product, TensorSpec
+from .base import MIXERS, POSITION_ENCODINGS, BiasedProduct, Mixer, PagedKVSpec, PartSpec, Product, TensorSpec
 
 
 @MIXERS.register("paged_gqa_attention")
@@ -350,13 +350,11 @@ class MixedHeadsAttention(NormedGQAAttention):
         table = step.block_tables[cache.group]
         proj = rt.buffer("amix_proj", n, self.w_in.rows, torch.float32)
         rt.gemm(x, self.w_in, proj)
-        if self.b_in is not None:
-            ops.add_rowvec(proj, self.b_in)
         q = rt.buffer("amix_q", n, H * P)
         ops.qkv_prepare(proj, self.cols, step.positions, step.tok_seq, table, q, cache.kv, H, D, Dv, 0, False, None,
                         self.q_gain, self.k_gain, self.qk_norm in ("head", "head_gain"), self.eps, write_cache=cache.writes,
                         row_scales=rt.buffer("amix_row_scales", n, 2, torch.float32) if self.qk_norm == "projection" else None,
-                        q_head_gain=self.q_head_gain, k_head_gain=self.k_head_gain)
+                        q_head_gain=self.q_head_gain, k_head_gain=self.k_head_gain, bias=self.b_in)      # (the biases are added as the projection is read)
         out = rt.buffer("amix_out", n, H * P)
         self.kernels.attention(q, out, cache.kv, step, table, H, self.scale, self.window, self.slopes, self.talk, self.sinks,
                                keep_first=self.keep_first, chunk=self.chunk)
@@ -364,8 +362,4 @@ class MixedHeadsAttention(NormedGQAAttention):
             packed = rt.buffer("amix_packed", n, H * Dv)
             ops.heads_gate(out, P, None, 0, None, packed, H)
             out = packed
-        if self.b_o is None:
-            return Product(out, self.w_o)
-        delta = rt.buffer("amix_delta", n, self.hidden_size, torch.float32)
-        rt.gemm(out, self.w_o, delta)
-        return ops.add_rowvec(delta, self.b_o)
+        return Product(out, self.w_o) if self.b_o is None else BiasedProduct(out, self.w_o, self.b_o)

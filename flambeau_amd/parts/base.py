@@ -285,6 +285,24 @@ class Product:
         return rt.gemm(self.x, self.weight, out)
 
 
+class BiasedProduct(Product):
+    """``x @ weight.T + bias`` (``bias`` float32, one value per output column).  Whoever only knows ``Product`` computes
+    product and bias apart; a receiver that adds a bias on its own way (the kernel that writes a sublayer's output into the
+    copies of a residual stream) takes ``product()`` and ``bias`` instead."""
+
+    def __init__(self, x, weight, bias):
+        super().__init__(x, weight)
+        self.bias = bias
+
+    def product(self, rt, out=None):
+        """The product alone."""
+        return super().compute(rt, out)
+
+    def compute(self, rt, out=None):
+        from ..kernels import ops
+        return ops.add_rowvec(super().compute(rt, out), self.bias)
+
+
 class Norm(Part):
     def forward(self, x, out, delta=None, store_sum=False, rows=None):
         """``out = norm(x (+ delta))``; ``x`` is the 32-bit residual stream; with

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartSpec, Product, TensorSpec
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BiasedProduct, Block, PartSpec, Product, TensorSpec
 from .norm import RMSNorm
 
 
@@ -62,7 +62,7 @@ class ResidualStream:
         """The normed stream in the compute dtype, the pending delta added on the way.  With
         ``lazy`` the caller takes what ``Norm.after_product`` returns as well as a tensor."""
         n, H = self.resid.shape
-        if lazy and rows is None and isinstance(self.pending, Product):
+        if lazy and rows is None and type(self.pending) is Product:          # (a product with a bias is computed first)
             fused = norm.after_product(self.rt, self.resid, self.pending)
             if fused is not None:
                 self.pending = None
@@ -99,14 +99,14 @@ class HyperStream(ResidualStream):
     def sublayer_input(self, in_w, norm, name="normed"):
         """norm(sum_s in_w[s] x_s) in the compute dtype; the waiting output of the sublayer before is written on the way."""
         n, W = self.resid.shape
-        y, mix, out_w = self.waiting if self.waiting is not None else (None, None, None)
+        y, mix, out_w, y_bias = self.waiting if self.waiting is not None else (None, None, None, None)
         u = self.rt.buffer("hyper_u", n, W, torch.float32)
         out = self.rt.buffer(name, n, W)
         if isinstance(norm, RMSNorm):
-            ops.hyper_step(self.copies, self.n_streams, y=y, mix=mix, out_w=out_w, in_w=in_w, u_out=u, gain=norm.weight,
+            ops.hyper_step(self.copies, self.n_streams, y=y, y_bias=y_bias, mix=mix, out_w=out_w, in_w=in_w, u_out=u, gain=norm.weight,
                            eps=norm.eps, normed=out)
         else:
-            ops.hyper_step(self.copies, self.n_streams, y=y, mix=mix, out_w=out_w, in_w=in_w, u_out=u)
+            ops.hyper_step(self.copies, self.n_streams, y=y, y_bias=y_bias, mix=mix, out_w=out_w, in_w=in_w, u_out=u)
             norm.forward(u, out)
         if y is not None:
             self.summed = False
@@ -117,13 +117,16 @@ class HyperStream(ResidualStream):
         """``delta``: what a part returned, a tensor or a ``Product``."""
         if self.waiting is not None:
             self._write()
-        if isinstance(delta, Product):
+        bias = None
+        if isinstance(delta, BiasedProduct):             # (its bias rides in the kernel that writes the copies)
+            delta, bias = delta.product(self.rt), delta.bias
+        elif isinstance(delta, Product):
             delta = delta.compute(self.rt)
-        self.waiting = (delta, mix, out_w)
+        self.waiting = (delta, mix, out_w, bias)
 
     def _write(self):
-        y, mix, out_w = self.waiting
-        ops.hyper_step(self.copies, self.n_streams, y=y, mix=mix, out_w=out_w)
+        y, mix, out_w, y_bias = self.waiting
+        ops.hyper_step(self.copies, self.n_streams, y=y, y_bias=y_bias, mix=mix, out_w=out_w)
         self.waiting, self.summed = None, False
 
     def flush(self):
@@ -131,8 +134,8 @@ class HyperStream(ResidualStream):
         if self.pending is not None:
             raise RuntimeError("a residual stream in several copies takes a sublayer's output with its numbers (sublayer_output), not a plain sum")
         if self.waiting is not None or not self.summed:
-            y, mix, out_w = self.waiting if self.waiting is not None else (None, None, None)
-            ops.hyper_step(self.copies, self.n_streams, y=y, mix=mix, out_w=out_w, in_w=self.ones, u_out=self.resid)
+            y, mix, out_w, y_bias = self.waiting if self.waiting is not None else (None, None, None, None)
+            ops.hyper_step(self.copies, self.n_streams, y=y, y_bias=y_bias, mix=mix, out_w=out_w, in_w=self.ones, u_out=self.resid)
             self.waiting, self.summed, self.cast = None, True, None
         return self.resid
 

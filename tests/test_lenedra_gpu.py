@@ -86,9 +86,10 @@ def test_hyper_connections_alone(dtype, S, W):
     want_u = np.tensordot(t2["in"].double().numpy(), copies, axes=(0, 0))
     assert np.abs(u.double().cpu().numpy() - want_u).max() < 3e-6 * size(t2["in"])
     assert np.abs(h.double().cpu().numpy() - pl.rms_norm(want_u, gain.double().numpy(), eps)).max() < tol * 4 * (1 + S / 4)
-    ops.hyper_step(xs, S, y=dev(y2), mix=dev(t2["mix"]), out_w=dev(t2["out"]))
+    bias = torch.randn(W, generator=g)                 # (a bias of the sublayer's last product rides in the same kernel)
+    ops.hyper_step(xs, S, y=dev(y2), y_bias=dev(bias), mix=dev(t2["mix"]), out_w=dev(t2["out"]))
     plain = {"p.in": t2["in"].double().numpy(), "p.out": t2["out"].double().numpy(), "p.mix": t2["mix"].double().numpy()}
-    copies = pl.hyper_sublayer(copies, plain, "p.", np.zeros(W), eps, lambda _: y2.double().numpy())
+    copies = pl.hyper_sublayer(copies, plain, "p.", np.zeros(W), eps, lambda _: (y2 + bias).double().numpy())
     total = torch.empty(n, W, device=DEV)
     ops.hyper_step(xs, S, in_w=torch.ones(S, device=DEV), u_out=total)
     assert np.abs(total.double().cpu().numpy() - copies.sum(axis=0)).max() < 3e-6 * S * np.abs(copies).max()
